@@ -144,7 +144,15 @@ class PyBlockPool:
 
 class BlockManager:
     def __init__(self, num_blocks: int, block_size: int = 16, watermark: float = 0.01,
-                 use_native: bool = True, prefix_caching: bool = True):
+                 use_native: bool = True, prefix_caching: bool = True, state_slots: int = 0):
+        """``state_slots`` > 0: the model keeps a recurrent state per sequence; every admitted
+        sequence also holds one of that many slots (freed with its blocks, lowest free slot
+        first).  A recurrent state summarises the whole prefix, so cached prefix blocks cannot
+        stand in for it: prefix caching is off for such models."""
+        self.state_slots = state_slots
+        self._free_slots = list(range(state_slots - 1, -1, -1))
+        if state_slots:
+            prefix_caching = False
         self.block_size = block_size
         self.num_blocks = num_blocks
         nat = _native() if use_native else None
@@ -194,17 +202,21 @@ class BlockManager:
         hit = self.pool.peek(hs) if hs else 0
         idle = self.pool.peek_idle(hs) if hit else 0
         need = self.blocks_needed(seq.num_tokens + 1) - hit
+        if self.state_slots and not self._free_slots:
+            return False
         return self.pool.num_free - need - idle >= self.watermark_blocks
 
     def allocate(self, seq: Sequence) -> bool:
         hs = self._prefix_hashes(seq)
         matched = self.pool.match(hs) if hs else []
         need = self.blocks_needed(seq.num_tokens + 1) - len(matched)
-        got = self.pool.allocate(need)
+        got = self.pool.allocate(need) if not (self.state_slots and not self._free_slots) else None
         if got is None:
             if matched:
                 self.pool.release(matched)
             return False
+        if self.state_slots:
+            seq.state_slot = self._free_slots.pop()
         seq.block_table = list(matched) + list(got)
         seq.num_cached = len(matched) * self.block_size
         seq.num_computed = seq.num_cached
@@ -221,6 +233,27 @@ class BlockManager:
         for i in range(seq.num_cached // self.block_size, min(len(hs), n_tokens // self.block_size)):
             self.pool.publish(seq.block_table[i], hs[i])
 
+    def admit(self, seq: Sequence) -> bool:
+        """Admit ``seq`` with no blocks yet (a caller that feeds it piecewise grows it with
+        :meth:`ensure_tokens`): takes its state slot where the model has recurrent state."""
+        if self.state_slots:
+            if not self._free_slots:
+                return False
+            seq.state_slot = self._free_slots.pop()
+        seq.num_cached = seq.num_computed = 0
+        seq.prefilled = False
+        return True
+
+    def ensure_tokens(self, seq: Sequence, n_tokens: int) -> bool:
+        """Grow seq's block table to hold ``n_tokens`` tokens."""
+        need = self.blocks_needed(n_tokens)
+        while len(seq.block_table) < need:
+            got = self.pool.allocate(1)
+            if got is None:
+                return False
+            seq.block_table.append(got[0])
+        return True
+
     def ensure_slot(self, seq: Sequence) -> bool:
         """Make room for the token at position seq.num_tokens (the next decode write)."""
         need = self.blocks_needed(seq.num_tokens + 1)
@@ -235,6 +268,10 @@ class BlockManager:
         if seq.block_table:
             self.pool.release(list(seq.block_table))
             seq.block_table = []
+        if seq.state_slot >= 0:
+            self._free_slots.append(seq.state_slot)
+            self._free_slots.sort(reverse=True)
+            seq.state_slot = -1
         seq.num_cached = 0
         seq.num_computed = 0
         seq.chunk = 0

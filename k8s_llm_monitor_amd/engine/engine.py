@@ -26,9 +26,8 @@ from typing import Optional, Union
 
 import torch
 
-from ..models.checkpoint import config_from_hf, load_checkpoint
 from ..models.config import ModelConfig, get_config
-from ..models.llama import CausalLM
+from ..models.registry import build_model, config_from_dir
 from ..parallel.state import ParallelState, get_state, serving_timeouts
 from ..parallel.step_bus import KIND_DECODE, KIND_PICKLE, KIND_STOP, bus_slot_bytes, decode_message, make_step_bus
 from ..parallel.health import PeerMonitor, gather_identities
@@ -69,6 +68,7 @@ class EngineConfig:
     # a Hugging Face model directory (config.json, *.safetensors, optional tokenizer.json): real
     # weights instead of the seeded random init (models/checkpoint.py); None = random init
     weights: Optional[str] = None
+    keep_logits: bool = False  # keep each step's logits on the device (trace replay; RunnerConfig.keep_logits)
 
 
 class _View:
@@ -95,20 +95,19 @@ class LLMEngine:
                 "cuda" if torch.cuda.is_available() else "cpu")
         self.device = torch.device(device)
         if model_cfg is None and cfg.weights:
-            model_cfg = config_from_hf(cfg.weights)
+            model_cfg = config_from_dir(cfg.weights)
         mc = model_cfg or get_config(cfg.model)
         if cfg.model_overrides:
             mc = mc.replace(**cfg.model_overrides)
         self.model_cfg = mc
         t0 = time.perf_counter()
-        self.model = CausalLM(mc, device=self.device, dtype=getattr(torch, cfg.dtype), seed=cfg.seed, pstate=self.ps,
-                              init="empty" if cfg.weights else "random")
-        if cfg.weights:
-            load_checkpoint(self.model, cfg.weights)
+        self.model = build_model(mc, device=self.device, dtype=getattr(torch, cfg.dtype), seed=cfg.seed,
+                                 pstate=self.ps, weights=cfg.weights)
         self.runner = ModelRunner(self.model, RunnerConfig(
             max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len, kv_cache_gb=cfg.kv_cache_gb,
-            num_blocks=cfg.num_blocks, use_graphs=cfg.use_graphs, seed=cfg.seed))
-        self.blocks = BlockManager(self.runner.num_blocks, prefix_caching=cfg.prefix_caching)
+            num_blocks=cfg.num_blocks, use_graphs=cfg.use_graphs, seed=cfg.seed, keep_logits=cfg.keep_logits))
+        self.blocks = BlockManager(self.runner.num_blocks, prefix_caching=cfg.prefix_caching,
+                                   state_slots=self.runner.num_state_slots)
         self.sched = Scheduler(SchedulerConfig(max_num_seqs=cfg.max_num_seqs,
                                                max_prefill_tokens=cfg.max_prefill_tokens,
                                                max_model_len=self.runner.max_len,

@@ -36,6 +36,9 @@ class RunnerConfig:
     num_blocks: Optional[int] = None  # overrides kv_cache_gb
     use_graphs: bool = True
     seed: int = 0
+    # keep every step's logits on the device (ModelRunner.last_logits / DecodeHandle.logits): the
+    # trace replayer reads them; serving leaves it off
+    keep_logits: bool = False
 
 
 class ModelRunner:
@@ -46,8 +49,15 @@ class ModelRunner:
         c = model.cfg
         self.max_len = min(cfg.max_model_len, c.max_position)
         self.max_blocks_per_seq = (self.max_len + BLOCK_SIZE - 1) // BLOCK_SIZE
-        L, hkv, D = c.n_layers, model.hkv, model.D
-        per_block = 2 * L * hkv * D * BLOCK_SIZE * 2  # bytes (K + V, bf16)
+        # layer-list models (models/hybrid.py) describe their own per-run caches: paged K / V for
+        # attention runs, per-sequence state slots for recurrent runs
+        self.hybrid = hasattr(model, "new_cache")
+        if self.hybrid:
+            per_block, per_slot = model.cache_bytes()
+            per_block = max(1, per_block)
+        else:
+            L, hkv, D = c.n_layers, model.hkv, model.D
+            per_block = 2 * L * hkv * D * BLOCK_SIZE * 2  # bytes (K + V, bf16)
         if cfg.num_blocks:
             nb = cfg.num_blocks
         elif cfg.kv_cache_gb <= 0:  # auto: every admitted sequence can reach max_len (+ one spare block)
@@ -55,9 +65,14 @@ class ModelRunner:
         else:
             nb = max(self.max_blocks_per_seq + 1, int(cfg.kv_cache_gb * (1 << 30) // per_block))
         self.num_blocks = nb
-        self.k_cache = torch.zeros(L, nb, hkv, D // 8, BLOCK_SIZE, 8, dtype=model.dtype, device=self.device)
-        self.v_cache = torch.zeros(L, nb, hkv, D, BLOCK_SIZE, dtype=model.dtype, device=self.device)
-        self.kv = [(self.k_cache[i], self.v_cache[i]) for i in range(L)]
+        self.num_state_slots = cfg.max_num_seqs if self.hybrid and model.has_state else 0
+        if self.hybrid:
+            self.k_cache = self.v_cache = None
+            self.kv = model.new_cache(nb, max(1, self.num_state_slots))
+        else:
+            self.k_cache = torch.zeros(L, nb, hkv, D // 8, BLOCK_SIZE, 8, dtype=model.dtype, device=self.device)
+            self.v_cache = torch.zeros(L, nb, hkv, D, BLOCK_SIZE, dtype=model.dtype, device=self.device)
+            self.kv = [(self.k_cache[i], self.v_cache[i]) for i in range(L)]
         self.is_gpu = self.device.type == "cuda"
         B = cfg.max_num_seqs
         self.B = B
@@ -66,14 +81,18 @@ class ModelRunner:
         # host staging (_Staging), so a step's inputs go over in a single host-to-device copy
         self.d_all = torch.zeros(_Staging.size(B, self.max_blocks_per_seq), dtype=torch.int32, device=dev)
         (self.d_ids, self.d_src, self.d_pos, self.d_slots, self.d_lens, self.d_topk, self.d_temp, self.d_topp,
-         self.d_bt) = _Staging.views(self.d_all, B, self.max_blocks_per_seq)
+         self.d_state, self.d_bt) = _Staging.views(self.d_all, B, self.max_blocks_per_seq)
         self.d_src.fill_(-1)
         self.d_slots.fill_(-1)
+        self.d_state.fill_(-1)
+        self.d_rows = torch.arange(B + 1, dtype=torch.int32, device=dev)  # decode rows as one-token segments
+        self.d_logits = None  # [B, vocab] fp32, the last decode step's logits (cfg.keep_logits)
+        self.last_logits = None
         self.d_topp.fill_(1.0)
         self.rng = torch.tensor([cfg.seed, 0], dtype=torch.int64, device=dev)
         self.d_out = torch.zeros(B, dtype=torch.int32, device=dev)
         self.decode_ws = ops.decode_workspace(B, model.hq, D, self.max_blocks_per_seq * BLOCK_SIZE, dev, model.hkv) \
-            if self.is_gpu else None
+            if self.is_gpu and not self.hybrid else None
         # pinned host staging, double-buffered: with pipelined decode the host fills step N+1's
         # inputs while step N's host-to-device copies may still be queued
         self.stage = [_Staging(B, self.max_blocks_per_seq, self.is_gpu, idx=i) for i in range(2)]
@@ -139,7 +158,8 @@ class ModelRunner:
             self._pf_bufs[i] = buf
         return buf
 
-    def prefill_launch(self, seqs: list[Sequence], decode: Optional[list] = None) -> "DecodeHandle":
+    def prefill_launch(self, seqs: list[Sequence], decode: Optional[list] = None,
+                       logit_rows: Optional[list] = None) -> "DecodeHandle":
         """Enqueue each sequence's scheduled prefill chunk - tokens [num_computed, num_computed +
         chunk) of its prompt (+ any tokens generated before a preemption) - without waiting for it;
         the first num_computed tokens already have their KV in the cache (prefix-cache hits,
@@ -148,7 +168,10 @@ class ModelRunner:
         first and attend through paged_decode.  The handle yields the sampled token of every decode
         row, then of every chunk (the first output token of the sequences whose prompt this step
         completes).  Every input goes over in ONE host-to-device copy from pinned memory, so a step
-        can be enqueued while the previous one still runs (pipelined prefill)."""
+        can be enqueued while the previous one still runs (pipelined prefill).
+        ``logit_rows`` (one list per decode row, then per chunk: offsets among that row's tokens of
+        this step): the step returns the logits at exactly those tokens in ``handle.logits``
+        ([n, vocab], in that order) and samples nothing (trace replay)."""
         dev = self.device
         decode = decode or []
         nd = len(decode)
@@ -161,7 +184,7 @@ class ModelRunner:
         cu[1:] = np.cumsum(lens)
         qs, st = ops.prefill_qblocks(cu.tolist(), ctx_starts=starts)
         nq = len(qs)
-        paged = any(starts)
+        paged = any(starts) or (self.hybrid and bool(seqs))  # layer-list attention always reads the pages
         W = max(len(s.block_table) for s in seqs) if paged else 0
         Wd = max(len(q.block_table) for q in decode) if nd else 0
         # TP > 1: two micro-batches of whole sequences, so one's row-parallel all-reduces overlap
@@ -174,7 +197,10 @@ class ModelRunner:
             mb = (ops.prefill_qblocks(cuA.tolist(), ctx_starts=starts[:kA]),
                   ops.prefill_qblocks(cuB.tolist(), ctx_starts=starts[kA:]))
         # layout of the staging buffer (int32 words; the float sampling parameters bit-cast)
-        sizes = dict(ids=T, pos=T, slots=T, cu=len(seqs) + 1, qs=nq, st=nq, lidx=R, temp=R, topk=R, topp=R,
+        nl = sum(len(x) for x in logit_rows) if logit_rows is not None else R
+        hy = R if self.hybrid else 0
+        sizes = dict(ids=T, pos=T, slots=T, cu=len(seqs) + 1, qs=nq, st=nq, lidx=nl, temp=R, topk=R, topp=R,
+                     gcu=hy + 1 if hy else 0, gctx=hy, gslot=hy,
                      cst=len(seqs) if paged else 0, bt=len(seqs) * W, dbt=nd * Wd, dlen=nd,
                      mcu=len(seqs) + 2 if kA else 0, mqs=nq if kA else 0, mst=nq if kA else 0,
                      mlidx=len(seqs) if kA else 0)
@@ -203,8 +229,18 @@ class ModelRunner:
         v["cu"][:] = cu
         v["qs"][:] = qs
         v["st"][:] = st
-        v["lidx"][:nd] = np.arange(nd, dtype=np.int32)
-        v["lidx"][nd:] = nd + cu[1:] - 1
+        if logit_rows is None:
+            v["lidx"][:nd] = np.arange(nd, dtype=np.int32)
+            v["lidx"][nd:] = nd + cu[1:] - 1
+        else:
+            first = np.concatenate([np.arange(nd, dtype=np.int32), nd + cu[:-1]])
+            v["lidx"][:] = [first[i] + k for i, ks in enumerate(logit_rows) for k in ks]
+        if hy:  # every row group as a segment of its sequence's recurrent state
+            v["gcu"][:nd + 1] = np.arange(nd + 1, dtype=np.int32)
+            v["gcu"][nd + 1:] = nd + cu[1:]
+            v["gctx"][:nd] = [q.num_tokens - 1 for q in decode]
+            v["gctx"][nd:] = starts
+            v["gslot"][:] = [getattr(q, "state_slot", -1) for q in rows]
         v["temp"].view(np.float32)[:] = [s.params.temperature for s in rows]
         v["topk"][:] = [s.params.top_k for s in rows]
         v["topp"].view(np.float32)[:] = [s.params.top_p for s in rows]
@@ -235,6 +271,8 @@ class ModelRunner:
         if paged:
             meta.ctx_start = dv["cst"]
             meta.block_tables = dv["bt"].view(len(seqs), W)
+        if hy:
+            meta.seg_cu, meta.seg_ctx, meta.seg_slot = dv["gcu"], dv["gctx"], dv["gslot"]
         if kA:
             TA, S_ = int(cu[kA]), len(seqs)
             parts = []
@@ -259,8 +297,12 @@ class ModelRunner:
         self.n_steps["prefill_context_tokens"] = self.n_steps.get("prefill_context_tokens", 0) + sum(starts)
         self.n_steps["prefill_tokens"] = self.n_steps.get("prefill_tokens", 0) + T
         logits = self.model.forward(dv["ids"], meta, self.kv)
-        tok = self._sample(logits, dv["temp"].view(torch.float32), dv["topk"], dv["topp"].view(torch.float32))
+        if self.cfg.keep_logits:
+            self.last_logits = logits
         self.n_steps["prefill"] += 1
+        if logit_rows is not None:
+            return DecodeHandle(nl, None, [], logits=logits)
+        tok = self._sample(logits, dv["temp"].view(torch.float32), dv["topk"], dv["topp"].view(torch.float32))
         if self.on_launched is not None:  # TP: the custom-AR error flag, read back with the tokens
             self.on_launched()
         if not self.is_gpu:
@@ -282,7 +324,14 @@ class ModelRunner:
         meta = AttnMeta(is_prefill=False, positions=self.d_pos[:b], slot_mapping=self.d_slots[:b],
                         block_tables=self.d_bt[:b], seq_lens=self.d_lens[:b], decode_ws=self.decode_ws,
                         dec_src=self.d_src[:b], dec_prev=self.d_out)
+        if self.hybrid:  # one-token segments: the tokens before this one are its position
+            meta.seg_cu, meta.seg_ctx, meta.seg_slot = self.d_rows[:b + 1], self.d_pos[:b], self.d_state[:b]
         logits = self.model.forward(self.d_ids[:b], meta, self.kv)
+        if self.cfg.keep_logits:
+            if self.d_logits is None:
+                self.d_logits = torch.zeros(self.B, logits.shape[1], dtype=torch.float32, device=self.device)
+            self.d_logits[:b].copy_(logits)
+            self.last_logits = self.d_logits[:b]
         self._sample(logits, self.d_temp[:b], self.d_topk[:b], self.d_topp[:b], out=self.d_out[:b])
 
     def capture_graphs(self, buckets: Optional[list[int]] = None) -> None:
@@ -331,6 +380,7 @@ class ModelRunner:
         st = self.stage[self._stage_i]
         self._stage_i ^= 1
         ids, pos_a, slots, lens, src = st.n_ids, st.n_pos, st.n_slots, st.n_lens, st.n_src
+        state = st.n_state
         temp, topk, topp, bt_a = st.n_temp, st.n_topk, st.n_topp, st.n_bt
         bt_a[:b] = 0
         for i, s in enumerate(seqs):
@@ -342,6 +392,7 @@ class ModelRunner:
             pos_a[i] = pos
             slots[i] = bt[pos // BLOCK_SIZE] * BLOCK_SIZE + pos % BLOCK_SIZE
             lens[i] = pos + 1
+            state[i] = getattr(s, "state_slot", -1)
             bt_a[i, : len(bt)] = bt
             p = s.params
             temp[i] = p.temperature
@@ -353,6 +404,7 @@ class ModelRunner:
             pos_a[n:b] = 0
             slots[n:b] = -1
             lens[n:b] = 0
+            state[n:b] = -1
             temp[n:b] = 0
             topk[n:b] = 0
             topp[n:b] = 1
@@ -410,7 +462,10 @@ class ModelRunner:
         return handle.out[: handle.n].tolist()
 
     def memory_report(self) -> dict:
-        kv = (self.k_cache.numel() + self.v_cache.numel()) * self.k_cache.element_size()
+        if self.hybrid:
+            kv = sum(t.numel() * t.element_size() for c in self.kv for t in c.values())
+        else:
+            kv = (self.k_cache.numel() + self.v_cache.numel()) * self.k_cache.element_size()
         return {"kv_cache_bytes": kv, "kv_blocks": self.num_blocks, "block_size": BLOCK_SIZE,
                 "max_model_len": self.max_len, "graph_buckets": sorted(self.graphs)}
 
@@ -418,13 +473,13 @@ class ModelRunner:
 class _Staging:
     """Pinned host buffer for one decode step's inputs, with numpy views for cheap writes.
 
-    One int32 buffer holds every field - ids, src, pos, slots, lens, top_k, temperature and top_p
-    ([B] each; the two float fields bit-cast) followed by the block tables [B, max_blocks] - so the
+    One int32 buffer holds every field - ids, src, pos, slots, lens, top_k, temperature, top_p
+    and the recurrent-state slot ([B] each; the two float fields bit-cast) followed by the block tables [B, max_blocks] - so the
     step's inputs reach the device in ONE copy of the per-row fields plus the live block-table rows
     (nine separate small copies were nine blit kernels of ~4.6 us each in front of every decode
     graph replay)."""
 
-    NFIELDS = 8
+    NFIELDS = 9
 
     @staticmethod
     def size(B: int, max_blocks: int) -> int:
@@ -436,7 +491,7 @@ class _Staging:
 
     @staticmethod
     def views(buf, B: int, max_blocks: int) -> tuple:
-        """(ids, src, pos, slots, lens, topk, temp, topp, bt) views of a buffer (torch or numpy)."""
+        """(ids, src, pos, slots, lens, topk, temp, topp, state, bt) views of a buffer (torch or numpy)."""
         f = [buf[i * B:(i + 1) * B] for i in range(_Staging.NFIELDS)]
         as_f32 = (lambda a: a.view(torch.float32)) if isinstance(buf, torch.Tensor) else (lambda a: a.view(np.float32))
         f[6], f[7] = as_f32(f[6]), as_f32(f[7])
@@ -456,7 +511,8 @@ class _Staging:
         self.full[0] = KIND_DECODE
         self.raw = self.full[DECODE_HDR:]
         (self.n_ids, self.n_src, self.n_pos, self.n_slots, self.n_lens, self.n_topk, self.n_temp, self.n_topp,
-         self.n_bt) = self.views(self.raw, B, max_blocks)
+         self.n_state, self.n_bt) = self.views(self.raw, B, max_blocks)
+        self.n_state[:] = -1
 
     def message(self, n: int, b: int, n_el: int) -> np.ndarray:
         from ..parallel.step_bus import DECODE_HDR
@@ -471,6 +527,7 @@ class DecodeHandle:
     event: object  # torch.cuda.Event, None on the CPU
     out: object  # pinned host tensor (GPU) or the token list (CPU)
     prev_event: object = None  # the back-to-back predecessor's end event (ModelRunner._chain_event)
+    logits: object = None  # [n, vocab] device tensor of a step launched with logit_rows
 
     def gpu_ms(self) -> Optional[float]:
         """This step's GPU time (after the event completed), or None when not measurable."""

@@ -40,6 +40,7 @@ class Sequence:
     output_ids: list[int] = field(default_factory=list)
     status: SeqStatus = SeqStatus.WAITING
     block_table: list[int] = field(default_factory=list)
+    state_slot: int = -1  # recurrent-state slot (models with recurrent mixers), -1 = none
     finish_reason: Optional[str] = None
     # timing (seconds, time.perf_counter clock)
     t_arrival: float = field(default_factory=time.perf_counter)

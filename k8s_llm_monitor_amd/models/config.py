@@ -139,3 +139,164 @@ def get_config(name: str) -> ModelConfig:
     if key not in PRESETS:
         raise KeyError(f"unknown model preset {name!r}; known: {sorted(PRESETS)}")
     return PRESETS[key]
+
+
+# ----------------------------------------------------------------------------- layer-list models
+
+@dataclass(frozen=True)
+class MoESpec:
+    """Routed feed-forward: ``experts`` SwiGLU experts of width ``ff`` of which each token takes
+    ``top`` (weights = softmax over the chosen router logits), plus an optional shared expert of
+    width ``shared_ff`` scaled by a per-token sigmoid gate (0 = none)."""
+
+    experts: int
+    top: int
+    ff: int
+    shared_ff: int = 0
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One decoder layer of a :class:`HybridConfig`: a token mixer (``kind`` names an entry of
+    models/hybrid.py MIXERS, ``mixer`` holds that mixer's sizes and constants as sorted
+    (key, value) pairs so the spec stays hashable) and an optional feed-forward."""
+
+    kind: str
+    mixer: tuple
+    mlp: Optional[MoESpec] = None
+
+    @property
+    def m(self) -> dict:
+        return dict(self.mixer)
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    """A decoder given as an explicit list of layers (attention and recurrent mixers may
+    alternate in any order), optionally with a span of layers that runs several times with shared
+    weights.  ``arch`` selects the model class (models/registry.py)."""
+
+    name: str
+    arch: str
+    vocab_size: int
+    d_model: int
+    layers: tuple  # of LayerSpec
+    max_position: int = 2048
+    norm_eps: float = 1e-5
+    logit_scale: float = 1.0
+    loop: Optional[tuple] = None  # (start, stop, times): layers start .. stop-1 run `times` times
+    bos_id: int = 1
+    eos_ids: tuple = (2,)
+    extra: dict = field(default_factory=dict)
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(s.mlp is not None for s in self.layers)
+
+    def runs(self) -> list:
+        """Execution order as (layer index, pass number or -1, first layer of its pass)."""
+        n = len(self.layers)
+        if not self.loop:
+            return [(i, -1, False) for i in range(n)]
+        a, b, times = self.loop
+        out = [(i, -1, False) for i in range(a)]
+        for t in range(times):
+            out += [(i, t, i == a) for i in range(a, b)]
+        return out + [(i, -1, False) for i in range(b, n)]
+
+    def replace(self, **kw) -> "HybridConfig":
+        return dataclasses.replace(self, **kw)
+
+
+def _flat(d: dict, prefix: str = "") -> list:
+    out = []
+    for k, v in d.items():
+        if isinstance(v, dict):
+            out += _flat(v, prefix + k + ".")
+        else:
+            out.append((prefix + k, v))
+    return out
+
+
+def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig:
+    """A :class:`HybridConfig` from a layer-list ``config.json``: ``architecture``, ``vocab``,
+    ``width``, ``max_positions``, ``norm.eps``, ``logit_scale``, ``loop`` {start, stop, times} and
+    ``layers`` [{type, mixer {...}, mlp {kind, expert.ff, router.experts, router.top, shared.ff} |
+    null}].  Nested mixer keys are flattened with dots (``mask.size``)."""
+    layers = []
+    for spec in c["layers"]:
+        ml = spec.get("mlp")
+        moe = None
+        if ml is not None:
+            if ml.get("kind", "moe") != "moe":
+                raise ValueError(f"unsupported feed-forward kind {ml.get('kind')!r}")
+            sh = ml.get("shared")
+            moe = MoESpec(experts=int(ml["router"]["experts"]), top=int(ml["router"]["top"]),
+                          ff=int(ml["expert"]["ff"]), shared_ff=int(sh["ff"]) if sh else 0)
+        layers.append(LayerSpec(kind=spec["type"], mixer=tuple(sorted(_flat(spec.get("mixer") or {}))), mlp=moe))
+    lp = c.get("loop")
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else None
+    if loop and not (0 <= loop[0] < loop[1] <= len(layers) and loop[2] >= 1):
+        raise ValueError(f"bad loop {lp!r} for {len(layers)} layers")
+    V = int(c["vocab"])
+    return HybridConfig(name=name or str(c.get("architecture", "hybrid")).lower(),
+                        arch=str(c["architecture"]).lower(), vocab_size=V, d_model=int(c["width"]),
+                        layers=tuple(layers), max_position=int(c.get("max_positions", 2048)),
+                        norm_eps=float(c["norm"]["eps"]), logit_scale=float(c.get("logit_scale", 1.0)), loop=loop,
+                        bos_id=int(c.get("bos_id", min(1, V - 1))), eos_ids=tuple(c.get("eos_ids", (min(2, V - 1),))))
+
+
+def hybrid_config_to_dict(c: HybridConfig) -> dict:
+    """The inverse of :func:`hybrid_config_from_dict`."""
+    def nest(pairs):
+        out: dict = {}
+        for k, v in pairs:
+            cur = out
+            parts = k.split(".")
+            for p in parts[:-1]:
+                cur = cur.setdefault(p, {})
+            cur[parts[-1]] = v
+        return out
+
+    layers = []
+    for s in c.layers:
+        ml = None
+        if s.mlp is not None:
+            ml = {"kind": "moe", "expert": {"ff": s.mlp.ff}, "router": {"experts": s.mlp.experts, "top": s.mlp.top},
+                  "shared": {"ff": s.mlp.shared_ff} if s.mlp.shared_ff else None}
+        layers.append({"type": s.kind, "mixer": nest(s.mixer), "mlp": ml})
+    d = {"architecture": c.arch.capitalize(), "vocab": c.vocab_size, "width": c.d_model, "layers": layers,
+         "max_positions": c.max_position, "norm": {"eps": c.norm_eps}, "logit_scale": c.logit_scale,
+         "bos_id": c.bos_id, "eos_ids": list(c.eos_ids)}
+    if c.loop:
+        d["loop"] = {"start": c.loop[0], "stop": c.loop[1], "times": c.loop[2]}
+    return d
+
+
+def _attn(heads, kv_heads, dim, vdim, window, scale):
+    return LayerSpec("attention", tuple(sorted({"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                                                "mask.size": window, "scale": scale}.items())))
+
+
+def _ssm(heads, vdim, state, groups, conv, norm_groups):
+    return LayerSpec("mamba2", tuple(sorted({"heads": heads, "vdim": vdim, "state": state, "groups": groups,
+                                             "conv": conv, "norm_groups": norm_groups}.items())))
+
+
+def _with_mlp(s: LayerSpec, m: Optional[MoESpec]) -> LayerSpec:
+    return dataclasses.replace(s, mlp=m)
+
+
+# Small Dunesun-design model for CPU tests and GPU smoke runs (random weights): recurrent and
+# windowed-attention layers interleaved, layers 1..2 looped twice.
+DUNESUN_TINY = _reg(HybridConfig(
+    name="dunesun-tiny", arch="dunesun", vocab_size=512, d_model=128,
+    layers=(_with_mlp(_ssm(4, 32, 16, 2, 4, 2), MoESpec(4, 2, 64, 96)),
+            _with_mlp(_attn(4, 2, 32, 16, 24, 0.2), MoESpec(4, 2, 64, 0)),
+            _with_mlp(_ssm(2, 64, 32, 1, 3, 1), None),
+            _with_mlp(_attn(2, 2, 64, 64, 8, 0.125), MoESpec(6, 3, 32, 64))),
+    max_position=1024, loop=(1, 3, 2), logit_scale=1.5, bos_id=1, eos_ids=(2,)))

@@ -75,6 +75,11 @@ class AttnMeta:
     # TP > 1 prefill as two micro-batches of whole sequences: (meta of rows [0, TA), meta of rows
     # [TA, T), TA); their row-parallel all-reduces overlap each other's compute (_prefill_overlap)
     micro: Optional[tuple] = None
+    # recurrent mixers (models/hybrid.py): every sequence's rows of this step as a segment - row
+    # offsets [R+1], tokens already in its state [R], its state slot [R] (< 0: padding row)
+    seg_cu: Optional[torch.Tensor] = None
+    seg_ctx: Optional[torch.Tensor] = None
+    seg_slot: Optional[torch.Tensor] = None
 
 
 def _seed_for(name: str, seed: int) -> int:

@@ -1,0 +1,370 @@
+// PyTorch bindings of the layer-list decoders' kernels (_k8sllm_hybrid).  Validates tensors (every
+// shape the kernels index by is checked here, on the host), picks the current HIP stream (so every
+// op is hipGraph-capturable) and calls the C launchers.  Activations are bfloat16 or float32.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime.h>
+
+extern "C" {
+int k8sllm_hy_embed_pos(float* out, const int* ids, const int* positions, const void* emb, const void* pos,
+                        const int* src, const int* prev, long T, int d, int vocab, int max_pos, int f32, hipStream_t s);
+int k8sllm_hy_add_norm(void* out, float* residual, const void* a0, int t0, const void* a1, int t1, const void* a2,
+                       int t2, const float* vec, const float* w, long rows, int d, float eps, int one_plus, int f32,
+                       hipStream_t s);
+int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_stride, const float* w, long rows,
+                               int n, int groups, float eps, int f32, hipStream_t s);
+int k8sllm_hy_swiglu(void* out, const void* gu, long rows, int f, int f32, hipStream_t s);
+int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float* kw, float eps, long T, int nq,
+                            int nk, int nv, void* k_cache, void* v_cache, const int* slots, int f32, hipStream_t s);
+int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
+                             const int* cu, const int* ctx, const int* block_tables, int bt_stride, int S, long T,
+                             int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink, int f32,
+                             hipStream_t s);
+int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
+                            const int* block_tables, int bt_stride, const int* seq_lens, int B, int Hq, int G, int dk,
+                            int dv, int bs, float scale, int window, int sink, int f32, hipStream_t s);
+int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int C, const float* cw, const float* cb,
+                        int taps, void* state, const int* cu, const int* ctx, const int* slot, int S, long T, int f32,
+                        hipStream_t s);
+int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
+                       const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
+                       const int* slot, int S, int nh, int P, int N, int G, int f32, hipStream_t s);
+int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
+                     const float* bias, int E, int K, int rows_w, int f32, hipStream_t s);
+int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
+                           int E, long rows, int N, int Kd, long w_es, int swiglu, int f32, hipStream_t s);
+int k8sllm_hy_combine(float* out, const void* ys, const int* inv, const float* wts, const void* shared,
+                      const float* gate, long T, int K, int d, int f32, hipStream_t s);
+int k8sllm_moe_align(const int* topk_ids, long n, int E, int* expert_offsets, int* sorted_idx, int* inv_idx,
+                     hipStream_t s);
+}
+
+namespace {
+
+using torch::Tensor;
+using OptT = c10::optional<Tensor>;
+
+hipStream_t cur() { return c10::hip::getCurrentHIPStream().stream(); }
+void check(int rc, const char* what) { TORCH_CHECK(rc == 0, "k8sllm hybrid kernel launch failed: ", what, " rc=", rc); }
+
+// activation dtype: 1 = fp32, 0 = bf16
+int act(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda(), n, " must be a GPU tensor");
+  TORCH_CHECK(t.scalar_type() == torch::kBFloat16 || t.scalar_type() == torch::kFloat32, n, " must be bf16 or fp32");
+  return t.scalar_type() == torch::kFloat32;
+}
+void same(const Tensor& t, int f32, const char* n) { TORCH_CHECK(act(t, n) == f32, n, ": activation dtype mismatch"); }
+void f32c(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 && t.is_contiguous(), n, " must be contiguous fp32 on the GPU");
+}
+void i32c(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt32 && t.is_contiguous(), n, " must be contiguous int32 on the GPU");
+}
+const int* iptr(const OptT& t, const char* n) {
+  if (!t.has_value()) return nullptr;
+  i32c(*t, n);
+  return t->data_ptr<int>();
+}
+int any_dt(const OptT& t, int64_t numel, const char* n) {  // 0 none, 1 bf16, 2 fp32
+  if (!t.has_value()) return 0;
+  const int f = act(*t, n);
+  TORCH_CHECK(t->is_contiguous() && t->numel() == numel, n, " must be contiguous and match the residual");
+  return f ? 2 : 1;
+}
+
+void embed_pos(Tensor out, Tensor ids, Tensor positions, Tensor emb, OptT pos, OptT src, OptT prev) {
+  const int f = act(emb, "embed");
+  f32c(out, "out");
+  i32c(ids, "ids");
+  i32c(positions, "positions");
+  TORCH_CHECK(emb.dim() == 2 && emb.is_contiguous(), "embed [V, d]");
+  const int64_t T = ids.numel(), d = emb.size(1);
+  TORCH_CHECK(out.numel() == T * d && positions.numel() >= T, "embed_pos: sizes");
+  int maxp = 1;
+  if (pos.has_value()) {
+    same(*pos, f, "pos");
+    TORCH_CHECK(pos->dim() == 2 && pos->is_contiguous() && pos->size(1) == d, "pos [P, d]");
+    maxp = (int)pos->size(0);
+  }
+  const int* sp = iptr(src, "src");
+  const int* pp = iptr(prev, "prev");
+  TORCH_CHECK((sp == nullptr) == (pp == nullptr), "src and prev come together");
+  if (sp) {
+    TORCH_CHECK(src->numel() >= T && prev->numel() >= 1, "src / prev sizes");
+  }
+  check(k8sllm_hy_embed_pos(out.data_ptr<float>(), ids.data_ptr<int>(), positions.data_ptr<int>(), emb.data_ptr(),
+                            pos.has_value() ? pos->data_ptr() : nullptr, sp, pp, T, (int)d, (int)emb.size(0), maxp, f, cur()),
+        "embed_pos");
+}
+
+void add_norm(Tensor out, Tensor residual, OptT a0, OptT a1, OptT a2, OptT vec, Tensor w, double eps, bool one_plus) {
+  const int f = act(out, "out");
+  f32c(residual, "residual");
+  f32c(w, "w");
+  TORCH_CHECK(residual.dim() == 2 && out.is_contiguous() && out.numel() == residual.numel(), "add_norm: out shape");
+  const int64_t rows = residual.size(0), d = residual.size(1);
+  TORCH_CHECK(w.numel() == d, "add_norm: w [d]");
+  const int t0 = any_dt(a0, rows * d, "addend 0"), t1 = any_dt(a1, rows * d, "addend 1"), t2 = any_dt(a2, rows * d, "addend 2");
+  if (vec.has_value()) {
+    f32c(*vec, "vec");
+    TORCH_CHECK(vec->numel() == d, "add_norm: vec [d]");
+  }
+  check(k8sllm_hy_add_norm(out.data_ptr(), residual.data_ptr<float>(), t0 ? a0->data_ptr() : nullptr, t0,
+                           t1 ? a1->data_ptr() : nullptr, t1, t2 ? a2->data_ptr() : nullptr, t2,
+                           vec.has_value() ? vec->data_ptr<float>() : nullptr, w.data_ptr<float>(), rows, (int)d, (float)eps,
+                           one_plus, f, cur()),
+        "add_norm");
+}
+
+void gated_group_norm(Tensor out, Tensor y, Tensor proj, int64_t z_col, Tensor w, double eps, int64_t groups) {
+  const int f = act(out, "out");
+  same(proj, f, "proj");
+  f32c(y, "y");
+  f32c(w, "w");
+  TORCH_CHECK(y.dim() == 2 && proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == y.size(0), "gated_group_norm: rows");
+  const int64_t n = y.size(1);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == y.numel() && w.numel() == n && z_col >= 0 && z_col + n <= proj.size(1) &&
+                  groups >= 1 && n % groups == 0,
+              "gated_group_norm: shapes");
+  check(k8sllm_hy_gated_group_norm(out.data_ptr(), y.data_ptr<float>(),
+                                   (const char*)proj.data_ptr() + z_col * proj.element_size(), proj.stride(0),
+                                   w.data_ptr<float>(), y.size(0), (int)n, (int)groups, (float)eps, f, cur()),
+        "gated_group_norm");
+}
+
+void swiglu(Tensor out, Tensor gu) {
+  const int f = act(gu, "gu");
+  same(out, f, "out");
+  TORCH_CHECK(gu.dim() == 2 && gu.is_contiguous() && out.is_contiguous() && gu.size(1) % 2 == 0 &&
+                  out.numel() * 2 == gu.numel(),
+              "swiglu: shapes");
+  check(k8sllm_hy_swiglu(out.data_ptr(), gu.data_ptr(), gu.size(0), (int)(gu.size(1) / 2), f, cur()), "swiglu");
+}
+
+// pages [blocks, bs, width]
+void pages(const Tensor& c, int f, int64_t width, const char* n) {
+  same(c, f, n);
+  TORCH_CHECK(c.dim() == 3 && c.is_contiguous() && c.size(2) == width, n, " must be [blocks, block, heads*dim]");
+}
+
+void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int64_t G, int64_t dk, int64_t dv,
+                   OptT k_cache, OptT v_cache, OptT slots) {
+  const int f = act(qkv, "qkv");
+  f32c(qw, "qw");
+  f32c(kw, "kw");
+  const int64_t nq = Hq * dk, nk = G * dk, nv = G * dv;
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) == nq + nk + nv, "qkv [T, Hq*dk + G*dk + G*dv]");
+  TORCH_CHECK(qw.numel() == nq && kw.numel() == nk, "q / k norm weights");
+  void *kc = nullptr, *vc = nullptr;
+  const int* sp = nullptr;
+  if (k_cache.has_value()) {
+    TORCH_CHECK(v_cache.has_value() && slots.has_value(), "k_cache, v_cache and slot_mapping come together");
+    pages(*k_cache, f, nk, "k_cache");
+    pages(*v_cache, f, nv, "v_cache");
+    TORCH_CHECK(k_cache->size(0) == v_cache->size(0) && k_cache->size(1) == v_cache->size(1), "k / v pages differ");
+    sp = iptr(slots, "slot_mapping");
+    TORCH_CHECK(slots->numel() >= qkv.size(0), "slot_mapping [T]");
+    kc = k_cache->data_ptr();
+    vc = v_cache->data_ptr();
+  }
+  check(k8sllm_hy_qk_norm_cache(qkv.data_ptr(), qkv.stride(0), qw.data_ptr<float>(), kw.data_ptr<float>(), (float)eps,
+                                qkv.size(0), (int)nq, (int)nk, (int)nv, kc, vc, sp, f, cur()),
+        "qk_norm_cache");
+}
+
+void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor cu, Tensor ctx,
+                              Tensor block_tables, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
+                              int64_t window, bool sink) {
+  const int f = act(qkv, "qkv");
+  same(out, f, "out");
+  pages(k_cache, f, G * dk, "k_cache");
+  pages(v_cache, f, G * dv, "v_cache");
+  i32c(cu, "cu");
+  i32c(ctx, "ctx");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == torch::kInt32 && block_tables.dim() == 2 &&
+                  block_tables.stride(1) == 1,
+              "block_tables [S, W] int32");
+  const int64_t T = qkv.size(0), S = ctx.numel();
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= Hq * dk, "qkv rows");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * Hq * dv, "out [T, Hq*dv]");
+  TORCH_CHECK(cu.numel() == S + 1 && block_tables.size(0) >= S, "cu [S+1], block_tables [S, W]");
+  TORCH_CHECK(window >= 0 && G >= 1 && Hq % G == 0, "heads / window");
+  check(k8sllm_hy_window_prefill(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+                                 cu.data_ptr<int>(), ctx.data_ptr<int>(), block_tables.data_ptr<int>(),
+                                 (int)block_tables.stride(0), (int)S, T, (int)Hq, (int)G, (int)dk, (int)dv,
+                                 (int)k_cache.size(1), (float)scale, (int)window, sink, f, cur()),
+        "window_attention_prefill");
+}
+
+void window_attention_decode(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor block_tables,
+                             Tensor seq_lens, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
+                             int64_t window, bool sink) {
+  const int f = act(qkv, "qkv");
+  same(out, f, "out");
+  pages(k_cache, f, G * dk, "k_cache");
+  pages(v_cache, f, G * dv, "v_cache");
+  i32c(seq_lens, "seq_lens");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == torch::kInt32 && block_tables.dim() == 2 &&
+                  block_tables.stride(1) == 1,
+              "block_tables [B, W] int32");
+  const int64_t B = qkv.size(0);
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= Hq * dk, "qkv rows");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == B * Hq * dv, "out [B, Hq*dv]");
+  TORCH_CHECK(seq_lens.numel() >= B && block_tables.size(0) >= B, "seq_lens [B], block_tables [B, W]");
+  TORCH_CHECK(window >= 0 && G >= 1 && Hq % G == 0, "heads / window");
+  check(k8sllm_hy_window_decode(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+                                block_tables.data_ptr<int>(), (int)block_tables.stride(0), seq_lens.data_ptr<int>(),
+                                (int)B, (int)Hq, (int)G, (int)dk, (int)dv, (int)k_cache.size(1), (float)scale,
+                                (int)window, sink, f, cur()),
+        "window_attention_decode");
+}
+
+void segs(const Tensor& cu, const Tensor& ctx, const Tensor& slot) {
+  i32c(cu, "seg_cu");
+  i32c(ctx, "seg_ctx");
+  i32c(slot, "seg_slot");
+  TORCH_CHECK(cu.numel() == ctx.numel() + 1 && slot.numel() == ctx.numel(), "segments: cu [R+1], ctx [R], slot [R]");
+}
+
+void conv_silu(Tensor out, Tensor proj, int64_t col0, Tensor cw, Tensor cb, Tensor state, Tensor cu, Tensor ctx,
+               Tensor slot) {
+  const int f = act(proj, "proj");
+  same(out, f, "out");
+  same(state, f, "conv_state");
+  f32c(cw, "conv_w");
+  f32c(cb, "conv_b");
+  segs(cu, ctx, slot);
+  const int64_t T = proj.size(0), C = cw.size(0), taps = cw.size(1);
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && col0 >= 0 && col0 + C <= proj.size(1), "proj columns");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * C && cb.numel() == C, "conv_silu: out / bias");
+  TORCH_CHECK(state.dim() == 3 && state.is_contiguous() && state.size(2) == C && state.size(1) >= taps - 1 &&
+                  (taps == 1 || state.size(1) == taps - 1),
+              "conv_state [slots, taps-1, C]");
+  check(k8sllm_hy_conv_silu(out.data_ptr(), proj.data_ptr(), proj.stride(0), (int)col0, (int)C, cw.data_ptr<float>(),
+                            cb.data_ptr<float>(), (int)taps, state.data_ptr(), cu.data_ptr<int>(), ctx.data_ptr<int>(),
+                            slot.data_ptr<int>(), (int)ctx.numel(), T, f, cur()),
+        "conv_silu");
+}
+
+void ssm_scan(Tensor y, Tensor xbc, Tensor proj, int64_t dt_col, Tensor dt_bias, Tensor a_log, Tensor d_skip,
+              Tensor state, Tensor cu, Tensor ctx, Tensor slot, int64_t nh, int64_t P, int64_t N, int64_t G) {
+  const int f = act(xbc, "xbc");
+  same(proj, f, "proj");
+  f32c(y, "y");
+  f32c(dt_bias, "dt_bias");
+  f32c(a_log, "A_log");
+  f32c(d_skip, "D");
+  f32c(state, "ssm_state");
+  segs(cu, ctx, slot);
+  const int64_t T = xbc.size(0);
+  TORCH_CHECK(xbc.dim() == 2 && xbc.is_contiguous() && xbc.size(1) == nh * P + 2 * G * N, "xbc [T, nh*P + 2*G*N]");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(0) == T && dt_col >= 0 && dt_col + nh <= proj.size(1),
+              "proj dt columns");
+  TORCH_CHECK(y.numel() == T * nh * P && dt_bias.numel() == nh && a_log.numel() == nh && d_skip.numel() == nh, "ssm sizes");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == nh && state.size(2) == N && state.size(3) == P, "ssm_state [slots, nh, N, P]");
+  TORCH_CHECK(G >= 1 && nh % G == 0 && N <= 256, "ssm: groups / state size (<= 256)");
+  check(k8sllm_hy_ssm_scan(y.data_ptr<float>(), xbc.data_ptr(), proj.data_ptr(), proj.stride(0), (int)dt_col,
+                           dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), d_skip.data_ptr<float>(),
+                           state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(), slot.data_ptr<int>(),
+                           (int)ctx.numel(), (int)nh, (int)P, (int)N, (int)G, f, cur()),
+        "ssm_scan");
+}
+
+void moe_router(Tensor ids, Tensor wts, OptT gate, Tensor h, Tensor wr, Tensor bias, int64_t E, int64_t K) {
+  const int f = act(h, "h");
+  i32c(ids, "ids");
+  f32c(wts, "wts");
+  f32c(wr, "router weight");
+  f32c(bias, "router bias");
+  const int64_t T = h.size(0), d = h.size(1);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && wr.dim() == 2 && wr.size(1) == d, "router: h [T, d], wr [E(+1), d]");
+  TORCH_CHECK(wr.size(0) == E || wr.size(0) == E + 1, "router rows");
+  TORCH_CHECK(bias.numel() >= E && ids.numel() == T * K && wts.numel() == T * K, "router: bias / outputs");
+  TORCH_CHECK(E <= 256 && K >= 1 && K <= 16 && K <= E, "router: up to 256 experts, top 16");
+  float* gp = nullptr;
+  if (gate.has_value()) {
+    f32c(*gate, "gate");
+    TORCH_CHECK(gate->numel() == T && wr.size(0) == E + 1, "gate [T] needs the extra router row");
+    gp = gate->data_ptr<float>();
+  }
+  check(k8sllm_hy_router(ids.data_ptr<int>(), wts.data_ptr<float>(), gp, h.data_ptr(), T, (int)d, wr.data_ptr<float>(),
+                         bias.data_ptr<float>(), (int)E, (int)K, (int)wr.size(0), f, cur()),
+        "moe_router");
+}
+
+void moe_align(Tensor ids, int64_t E, Tensor offsets, Tensor sorted_idx, Tensor inv_idx) {
+  i32c(ids, "ids");
+  i32c(offsets, "offsets");
+  i32c(sorted_idx, "sorted_idx");
+  i32c(inv_idx, "inv_idx");
+  TORCH_CHECK(offsets.numel() == E + 1 && sorted_idx.numel() == ids.numel() && inv_idx.numel() == ids.numel() && E <= 256,
+              "moe_align sizes");
+  check(k8sllm_moe_align(ids.data_ptr<int>(), ids.numel(), (int)E, offsets.data_ptr<int>(), sorted_idx.data_ptr<int>(),
+                         inv_idx.data_ptr<int>(), cur()),
+        "moe_align");
+}
+
+// y [rows, N] = W[e] a over expert-sorted rows; sorted_idx given: a's row of sorted row r is sorted_idx[r] / div
+void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx, int64_t div, bool swiglu) {
+  const int f = act(a, "a");
+  same(y, f, "y");
+  same(w, f, "w");
+  i32c(offsets, "offsets");
+  TORCH_CHECK(a.dim() == 2 && a.is_contiguous() && w.dim() == 3 && w.is_contiguous() && y.dim() == 2 && y.is_contiguous(),
+              "grouped_gemm: layouts");
+  const int64_t E = w.size(0), Kd = w.size(2), rows = y.size(0);
+  const int64_t N = swiglu ? w.size(1) / 2 : w.size(1);
+  TORCH_CHECK(a.size(1) == Kd && y.size(1) == N && offsets.numel() == E + 1 && (!swiglu || w.size(1) % 2 == 0),
+              "grouped_gemm: shapes");
+  const int* sp = iptr(sorted_idx, "sorted_idx");
+  if (sp) {
+    TORCH_CHECK(sorted_idx->numel() == rows && div >= 1 && a.size(0) * div >= rows, "grouped_gemm: gather index");
+  } else {
+    TORCH_CHECK(a.size(0) == rows, "grouped_gemm: a rows");
+  }
+  check(k8sllm_hy_grouped_gemm(y.data_ptr(), a.data_ptr(), w.data_ptr(), offsets.data_ptr<int>(), sp, (int)div, (int)E,
+                               rows, (int)N, (int)Kd, w.size(1) * Kd, swiglu, f, cur()),
+        "grouped_gemm");
+}
+
+void moe_combine(Tensor out, Tensor ys, Tensor inv, Tensor wts, OptT shared, OptT gate) {
+  const int f = act(ys, "ys");
+  f32c(out, "out");
+  f32c(wts, "wts");
+  i32c(inv, "inv_idx");
+  const int64_t T = out.size(0), d = out.size(1), K = wts.numel() / std::max<int64_t>(T, 1);
+  TORCH_CHECK(out.dim() == 2 && ys.dim() == 2 && ys.is_contiguous() && ys.size(1) == d && ys.size(0) == T * K &&
+                  inv.numel() == T * K && wts.numel() == T * K,
+              "moe_combine: shapes");
+  const void* sh = nullptr;
+  const float* gp = nullptr;
+  if (shared.has_value()) {
+    same(*shared, f, "shared");
+    TORCH_CHECK(gate.has_value() && shared->is_contiguous() && shared->numel() == T * d, "shared [T, d] with its gate");
+    f32c(*gate, "gate");
+    TORCH_CHECK(gate->numel() == T, "gate [T]");
+    sh = shared->data_ptr();
+    gp = gate->data_ptr<float>();
+  }
+  check(k8sllm_hy_combine(out.data_ptr<float>(), ys.data_ptr(), inv.data_ptr<int>(), wts.data_ptr<float>(), sh, gp, T,
+                          (int)K, (int)d, f, cur()),
+        "moe_combine");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("embed_pos", &embed_pos);
+  m.def("add_norm", &add_norm);
+  m.def("gated_group_norm", &gated_group_norm);
+  m.def("swiglu", &swiglu);
+  m.def("qk_norm_cache", &qk_norm_cache);
+  m.def("window_attention_prefill", &window_attention_prefill);
+  m.def("window_attention_decode", &window_attention_decode);
+  m.def("conv_silu", &conv_silu);
+  m.def("ssm_scan", &ssm_scan);
+  m.def("moe_router", &moe_router);
+  m.def("moe_align", &moe_align);
+  m.def("grouped_gemm", &grouped_gemm);
+  m.def("moe_combine", &moe_combine);
+}

@@ -1,0 +1,213 @@
+// Routed feed-forward of the layer-list decoders (any sizes, bf16 or fp32 activations).
+//   moe_router    fp32 logits = Wr h + b (h widened from its storage dtype), the K largest chosen
+//                 (lowest index wins a tie), weights = softmax over the chosen logits only; one
+//                 more row of Wr, if present, gives gate = sigmoid(Wr[E] h) (the shared expert's)
+//   grouped_gemm  Y[r] = W[e(r)] A[row(r)] over expert-sorted rows r (offsets / sorted_idx from the
+//                 counting sort), the A rows gathered on load; SWIGLU: W = [gate rows ; up rows] and
+//                 Y = silu(gate) * up.  64 x 64 tiles, fp32 accumulation.
+//   moe_combine   out[t] = sum_k w[t][k] Y[inv[t*K + k]] + gate[t] * shared[t]   (fp32)
+#include "hy_common.h"
+
+namespace k8sllm {
+
+constexpr int kMaxE = 256;
+constexpr int kMaxK = 16;
+
+template <typename T>
+__global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, float* __restrict__ wts,
+                                                        float* __restrict__ gate, const T* __restrict__ h, int d,
+                                                        const float* __restrict__ wr, const float* __restrict__ bias,
+                                                        int E, int K, int rows_w) {
+  __shared__ float lg[kMaxE + 1];
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* x = h + t * d;
+  for (int e = wave; e < rows_w; e += 4) {
+    const float* w = wr + (long)e * d;
+    float a = 0.f;
+    for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
+    a = wave_sum(a);
+    if (lane == 0) lg[e] = e < E ? a + bias[e] : a;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sel[kMaxK];
+    float val[kMaxK];
+    float mx = -INFINITY;
+    for (int k = 0; k < K; ++k) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e) {
+        bool taken = false;
+        for (int j = 0; j < k; ++j) taken |= sel[j] == e;
+        if (!taken && (best < 0 || lg[e] > bv)) {
+          bv = lg[e];
+          best = e;
+        }
+      }
+      sel[k] = best;
+      val[k] = bv;
+      mx = fmaxf(mx, bv);
+    }
+    float z = 0.f;
+    for (int k = 0; k < K; ++k) {
+      val[k] = expf(val[k] - mx);
+      z += val[k];
+    }
+    for (int k = 0; k < K; ++k) {
+      ids[t * K + k] = sel[k];
+      wts[t * K + k] = val[k] / z;
+    }
+    if (gate != nullptr) gate[t] = 1.f / (1.f + expf(-lg[E]));
+  }
+}
+
+constexpr int TM = 64, TN = 64, TK = 16;
+
+template <typename T, bool SWIGLU>
+__global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y, const T* __restrict__ A,
+                                                              const T* __restrict__ W, const int* __restrict__ offsets,
+                                                              const int* __restrict__ sorted_idx, int div, int E,
+                                                              int N, int Kd, long w_es) {
+  __shared__ float As[TK][TM + 4];
+  __shared__ float Ws[TK][TN + 4];
+  __shared__ float Us[SWIGLU ? TK : 1][TN + 4];
+  // this workgroup's (expert, row tile): tiles are numbered expert by expert
+  int e = 0, tile = blockIdx.x, r0 = 0, r1 = 0;
+  for (; e < E; ++e) {
+    r0 = offsets[e];
+    r1 = offsets[e + 1];
+    const int nt = (r1 - r0 + TM - 1) / TM;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (e >= E) return;
+  r0 += tile * TM;
+  const int n0 = blockIdx.y * TN;
+  const T* We = W + (long)e * w_es;
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;  // 4 x 4 outputs per thread: rows ty*4.., cols tx*4..
+  float acc[4][4], accu[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = accu[i][j] = 0.f;
+  // loader: thread -> (row lr, k offsets lk, lk + 4, ...) of the 64 x 16 tiles
+  const int lr = tid >> 2, lk = (tid & 3) * 4;
+  const int arow = r0 + lr;
+  long asrc = -1;
+  if (arow < r1) asrc = sorted_idx != nullptr ? sorted_idx[arow] / div : arow;
+  const int wrow = n0 + lr;
+  for (int k0 = 0; k0 < Kd; k0 += TK) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + lk + j;
+      As[lk + j][lr] = (asrc >= 0 && k < Kd) ? ldf(A + asrc * Kd + k) : 0.f;
+      Ws[lk + j][lr] = (wrow < N && k < Kd) ? ldf(We + (long)wrow * Kd + k) : 0.f;
+      if (SWIGLU) Us[lk + j][lr] = (wrow < N && k < Kd) ? ldf(We + (long)(N + wrow) * Kd + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < TK; ++k) {
+      float a[4], b[4], u[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Ws[k][tx * 4 + j];
+      if (SWIGLU) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) u[j] = Us[k][tx * 4 + j];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] += a[i] * b[j];
+          if (SWIGLU) accu[i][j] += a[i] * u[j];
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + ty * 4 + i;
+    if (r >= r1) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (SWIGLU) {
+        // the separate-projection form rounds gate and up to the storage dtype before the product
+        T gq, uq;
+        stf(&gq, v);
+        stf(&uq, accu[i][j]);
+        v = silu_f(ldf(&gq)) * ldf(&uq);
+      }
+      stf(Y + (long)r * N + n, v);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void hy_combine_kernel(float* __restrict__ out, const T* __restrict__ ys,
+                                                         const int* __restrict__ inv, const float* __restrict__ wts,
+                                                         const T* __restrict__ shared, const float* __restrict__ gate,
+                                                         int K, int d) {
+  const long t = blockIdx.x;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float a = 0.f;
+    for (int k = 0; k < K; ++k) a += wts[t * K + k] * ldf(ys + (long)inv[t * K + k] * d + c);
+    if (shared != nullptr) a += gate[t] * ldf(shared + t * d + c);
+    out[t * d + c] = a;
+  }
+}
+
+}  // namespace k8sllm
+
+using namespace k8sllm;
+
+extern "C" {
+
+int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
+                     const float* bias, int E, int K, int rows_w, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (E > kMaxE || K > kMaxK || K > E || K < 1 || rows_w < E || rows_w > E + 1) return -1;
+  if (f32)
+    hipLaunchKernelGGL(hy_router_kernel<float>, dim3(T), dim3(256), 0, s, ids, wts, gate, (const float*)h, d, wr, bias,
+                       E, K, rows_w);
+  else
+    hipLaunchKernelGGL(hy_router_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids, wts, gate, (const bf16_t*)h, d, wr,
+                       bias, E, K, rows_w);
+  return (int)hipGetLastError();
+}
+
+// rows: the sorted rows in all (an upper bound of the row tiles is rows / 64 + E)
+int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
+                           int E, long rows, int N, int Kd, long w_es, int swiglu, int f32, hipStream_t s) {
+  if (rows <= 0) return 0;
+  const dim3 grid((unsigned)(rows / TM + E), (unsigned)((N + TN - 1) / TN));
+#define K8SLLM_GG(T, SW)                                                                                            \
+  hipLaunchKernelGGL((hy_grouped_gemm_kernel<T, SW>), grid, dim3(256), 0, s, (T*)Y, (const T*)A, (const T*)W, offsets, \
+                     sorted_idx, div, E, N, Kd, w_es)
+  if (f32) {
+    if (swiglu) K8SLLM_GG(float, true); else K8SLLM_GG(float, false);
+  } else {
+    if (swiglu) K8SLLM_GG(bf16_t, true); else K8SLLM_GG(bf16_t, false);
+  }
+#undef K8SLLM_GG
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_combine(float* out, const void* ys, const int* inv, const float* wts, const void* shared,
+                      const float* gate, long T, int K, int d, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (f32)
+    hipLaunchKernelGGL(hy_combine_kernel<float>, dim3(T), dim3(256), 0, s, out, (const float*)ys, inv, wts,
+                       (const float*)shared, gate, K, d);
+  else
+    hipLaunchKernelGGL(hy_combine_kernel<bf16_t>, dim3(T), dim3(256), 0, s, out, (const bf16_t*)ys, inv, wts,
+                       (const bf16_t*)shared, gate, K, d);
+  return (int)hipGetLastError();
+}
+}

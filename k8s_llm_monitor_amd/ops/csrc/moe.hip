@@ -111,8 +111,10 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const bf16_t* __restric
 
 constexpr int kAT = 1024;
 constexpr int kMaxE = 16;
+constexpr int kAlignMaxE = 256;  // up to this many experts with fewer threads (same 64 KiB of counters)
 
-// exclusive scan of one value per thread over the 1024-thread workgroup
+// exclusive scan of one value per thread over an NT-thread workgroup
+template <int NT>
 __device__ __forceinline__ int block_exscan(int v, int* wsum, int& total) {
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   int x = v;
@@ -126,7 +128,7 @@ __device__ __forceinline__ int block_exscan(int v, int* wsum, int& total) {
   int pre = 0;
   total = 0;
 #pragma unroll
-  for (int i = 0; i < kAT / 64; ++i) {
+  for (int i = 0; i < NT / 64; ++i) {
     const int s = wsum[i];
     if (i < w) pre += s;
     total += s;
@@ -135,13 +137,16 @@ __device__ __forceinline__ int block_exscan(int v, int* wsum, int& total) {
   return pre + x - v;
 }
 
-__global__ __launch_bounds__(kAT) void moe_align_kernel(const int* __restrict__ ids, long n, int E,
-                                                        int* __restrict__ offsets, int* __restrict__ sorted_idx,
-                                                        int* __restrict__ inv_idx) {
-  __shared__ int cnt[kMaxE][kAT];
-  __shared__ int wsum[kAT / 64];
+// NT threads x ME experts of per-thread counters fill the 64 KiB of LDS: 1024 x 16 (Mixtral),
+// 256 x 64, 64 x 256.
+template <int NT, int ME>
+__global__ __launch_bounds__(NT) void moe_align_kernel(const int* __restrict__ ids, long n, int E,
+                                                       int* __restrict__ offsets, int* __restrict__ sorted_idx,
+                                                       int* __restrict__ inv_idx) {
+  __shared__ int cnt[ME][NT];
+  __shared__ int wsum[NT / 64];
   const int t = threadIdx.x;
-  const long C = (n + kAT - 1) / kAT;
+  const long C = (n + NT - 1) / NT;
   const long b0 = t * C, b1 = min(n, b0 + C);
   for (int e = 0; e < E; ++e) cnt[e][t] = 0;
   for (long i = b0; i < b1; ++i) cnt[ids[i]][t] += 1;
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(kAT) void moe_align_kernel(const int* __restrict__ 
   int base = 0;
   for (int e = 0; e < E; ++e) {
     int tot;
-    const int ex = block_exscan(cnt[e][t], wsum, tot);
+    const int ex = block_exscan<NT>(cnt[e][t], wsum, tot);
     if (t == 0) offsets[e] = base;
     cnt[e][t] = base + ex;  // start position of this thread's items of expert e
     base += tot;
@@ -219,8 +224,16 @@ int k8sllm_moe_router(const void* x, const void* wr, long T, int d, int E, int K
 
 int k8sllm_moe_align(const int* topk_ids, long n, int E, int* expert_offsets, int* sorted_idx, int* inv_idx,
                      hipStream_t s) {
-  if (E > kMaxE) return -1;
-  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(kAT), 0, s, topk_ids, n, E, expert_offsets, sorted_idx, inv_idx);
+  if (E > kAlignMaxE) return -1;
+  if (E <= kMaxE)
+    hipLaunchKernelGGL((moe_align_kernel<kAT, kMaxE>), dim3(1), dim3(kAT), 0, s, topk_ids, n, E, expert_offsets,
+                       sorted_idx, inv_idx);
+  else if (E <= 64)
+    hipLaunchKernelGGL((moe_align_kernel<256, 64>), dim3(1), dim3(256), 0, s, topk_ids, n, E, expert_offsets,
+                       sorted_idx, inv_idx);
+  else
+    hipLaunchKernelGGL((moe_align_kernel<64, kAlignMaxE>), dim3(1), dim3(64), 0, s, topk_ids, n, E, expert_offsets,
+                       sorted_idx, inv_idx);
   return (int)hipGetLastError();
 }
 

@@ -227,7 +227,7 @@ def decode_message(buf: bytes) -> tuple:
 def bus_slot_bytes(max_num_seqs: int, max_model_len: int, max_blocks: int) -> int:
     """Enough for the largest message: a raw decode step or a pickled prefill plan (chunk ids +
     block tables of every sequence)."""
-    raw = 4 * (DECODE_HDR + 8 * max_num_seqs + max_num_seqs * max_blocks)
+    raw = 4 * (DECODE_HDR + 9 * max_num_seqs + max_num_seqs * max_blocks)
     pickled = max_num_seqs * (max_model_len * 6 + max_blocks * 6 + 256) + (1 << 16)
     return int(max(1 << 20, raw, pickled))
 

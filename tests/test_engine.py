@@ -252,7 +252,7 @@ def test_decode_staging_layout_and_resolve_ids_cpu():
 
     B, mb = 8, 5
     st = _Staging(B, mb, pin=False)
-    assert st.h_all.numel() == _Staging.size(B, mb) == 8 * B + B * mb
+    assert st.h_all.numel() == _Staging.size(B, mb) == 9 * B + B * mb
     st.n_ids[:] = 1
     st.n_src[:] = 2
     st.n_pos[:] = 3
@@ -261,16 +261,17 @@ def test_decode_staging_layout_and_resolve_ids_cpu():
     st.n_topk[:] = 6
     st.n_temp[:] = 0.5
     st.n_topp[:] = 0.25
+    st.n_state[:] = 7
     st.n_bt[:] = 9
     raw = st.h_all.numpy()
     for i, v in enumerate([1, 2, 3, 4, 5, 6]):
         assert (raw[i * B:(i + 1) * B] == v).all()
     assert (raw[6 * B:7 * B].view(np.float32) == 0.5).all() and (raw[7 * B:8 * B].view(np.float32) == 0.25).all()
-    assert (raw[8 * B:] == 9).all()
-    assert _Staging.prefix(B, mb, 3) == 8 * B + 3 * mb
+    assert (raw[8 * B:9 * B] == 7).all() and (raw[9 * B:] == 9).all()
+    assert _Staging.prefix(B, mb, 3) == 9 * B + 3 * mb
     dev = torch.zeros(_Staging.size(B, mb), dtype=torch.int32)
     views = _Staging.views(dev, B, mb)
-    assert views[6].dtype == torch.float32 and views[8].shape == (B, mb)
+    assert views[6].dtype == torch.float32 and views[9].shape == (B, mb)
     ids = torch.tensor([10, 11, 12, 13], dtype=torch.int32)
     src = torch.tensor([-1, 2, -1, 0], dtype=torch.int32)
     prev = torch.tensor([100, 101, 102, 103], dtype=torch.int32)

@@ -1,0 +1,170 @@
+"""gfx950 kernels of the layer-list decoders (_k8sllm_hybrid) against the fp32 torch form of the
+same op, bf16 and fp32 activations, at sizes that are not multiples of the kernels' tiles."""
+import math
+
+import pytest
+import torch
+
+from k8s_llm_monitor_amd.ops import hybrid as H
+
+pytestmark = pytest.mark.gpu
+DT = [torch.float32, torch.bfloat16]
+
+
+def _tol(dt):
+    return dict(rtol=2e-5, atol=2e-5) if dt == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def _g(seed=0):
+    return torch.Generator().manual_seed(seed)
+
+
+def _r(g, *shape, s=1.0, dt=torch.float32):
+    return (torch.randn(*shape, generator=g) * s).to(dt)
+
+
+def _i32(x):
+    return torch.tensor(x, dtype=torch.int32)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_embed_pos_and_add_norm(dt):
+    g = _g(1)
+    V, d, T = 50, 72, 7
+    emb, pos = _r(g, V, d, dt=dt), _r(g, 40, d, dt=dt)
+    ids, p = torch.randint(0, V, (T,), generator=g, dtype=torch.int32), torch.randint(0, 40, (T,), generator=g, dtype=torch.int32)
+    src, prev = _i32([-1, 2, -1, 0, -1, -1, 1]), _i32([5, 6, 7])
+    want = H.embed_pos(ids, p, emb, pos, src, prev)
+    got = H.embed_pos(ids.cuda(), p.cuda(), emb.cuda(), pos.cuda(), src.cuda(), prev.cuda())
+    assert torch.equal(got.cpu(), want)
+    a, b, x0, vec, w = _r(g, T, d, dt=dt), _r(g, T, d), _r(g, T, d), _r(g, d), _r(g, d, s=0.2)
+    for one_plus, adds, v in ((True, (a, b, x0), vec), (False, (a,), None), (True, (), None)):
+        r_c, r_g = want.clone(), want.clone().cuda()
+        y_c = H.add_norm(r_c, adds, v, w, 1e-5, one_plus, dt)
+        y_g = H.add_norm(r_g, tuple(t.cuda() for t in adds), v.cuda() if v is not None else None, w.cuda(), 1e-5, one_plus, dt)
+        torch.testing.assert_close(r_g.cpu(), r_c, rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(y_g.cpu().float(), y_c.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_gated_group_norm_and_swiglu(dt):
+    g = _g(2)
+    T, n, groups = 5, 96, 3
+    y, proj, w = _r(g, T, n), _r(g, T, n + 40, dt=dt), _r(g, n, s=0.3) + 1
+    want = H.gated_group_norm(y, proj, 8, w, 1e-5, groups, dt)
+    got = H.gated_group_norm(y.cuda(), proj.cuda(), 8, w.cuda(), 1e-5, groups, dt)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+    gu = _r(g, T, 2 * 37, dt=dt)
+    torch.testing.assert_close(H.swiglu(gu.cuda()).cpu().float(), H.swiglu(gu).float(), **_tol(dt))
+
+
+def _paged(g, dt, lens, Hq, G, dk, dv, nb=40, bs=16, shuffle=True):
+    """Random q rows and a paged cache holding ``lens`` tokens per sequence on shuffled pages."""
+    perm = torch.randperm(nb, generator=g).tolist() if shuffle else list(range(nb))
+    W = max((n + bs - 1) // bs for n in lens)
+    bt = torch.zeros(len(lens), W, dtype=torch.int32)
+    kc, vc = _r(g, nb, bs, G * dk, dt=dt), _r(g, nb, bs, G * dv, dt=dt)
+    for s, n in enumerate(lens):
+        for j in range((n + bs - 1) // bs):
+            bt[s, j] = perm.pop()
+    return kc, vc, bt
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("window,sink", [(5, True), (0, True), (70, False), (16, True)])
+def test_window_attention_kernels(dt, window, sink):
+    g = _g(3)
+    Hq, G, dk, dv = 6, 2, 24, 40
+    ctx, new = [0, 37, 130], [9, 20, 3]
+    lens = [c + n for c, n in zip(ctx, new)]
+    kc, vc, bt = _paged(g, dt, lens, Hq, G, dk, dv)
+    cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
+    qkv = _r(g, sum(new), Hq * dk + G * (dk + dv), dt=dt)
+    a = (Hq, G, dk, dv, 0.3, window, sink)
+    want = H.window_attention_prefill(qkv, kc, vc, cu, _i32(ctx), bt, *a)
+    got = H.window_attention_prefill(qkv.cuda(), kc.cuda(), vc.cuda(), cu.cuda(), _i32(ctx).cuda(), bt.cuda(), *a)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+    # decode: one query per sequence (plus a padding row of length 0)
+    q1 = _r(g, 4, Hq * dk + G * (dk + dv), dt=dt)
+    sl = _i32(lens + [0])
+    bt4 = torch.cat([bt, torch.zeros(1, bt.shape[1], dtype=torch.int32)])
+    want = H.window_attention_decode(q1, kc, vc, bt4, sl, *a)
+    got = H.window_attention_decode(q1.cuda(), kc.cuda(), vc.cuda(), bt4.cuda(), sl.cuda(), *a)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_qk_norm_cache(dt):
+    g = _g(4)
+    Hq, G, dk, dv, T = 3, 1, 20, 12, 6
+    qkv = _r(g, T, Hq * dk + G * (dk + dv), dt=dt)
+    qw, kw = _r(g, Hq * dk, s=0.3) + 1, _r(g, G * dk, s=0.3) + 1
+    slots = _i32([17, 3, -1, 40, 41, 0])
+    kc, vc = torch.zeros(4, 16, G * dk, dtype=dt), torch.zeros(4, 16, G * dv, dtype=dt)
+    a_c, a_g = qkv.clone(), qkv.clone().cuda()
+    kg, vg = kc.clone().cuda(), vc.clone().cuda()
+    H.qk_norm_cache(a_c, qw, kw, 1e-5, Hq, G, dk, dv, kc, vc, slots)
+    H.qk_norm_cache(a_g, qw.cuda(), kw.cuda(), 1e-5, Hq, G, dk, dv, kg, vg, slots.cuda())
+    torch.testing.assert_close(a_g.cpu().float(), a_c.float(), **_tol(dt))
+    torch.testing.assert_close(kg.cpu().float(), kc.float(), **_tol(dt))
+    torch.testing.assert_close(vg.cpu().float(), vc.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("taps", [1, 2, 4])
+def test_conv_silu_with_state(dt, taps):
+    g = _g(5)
+    C, col0 = 70, 9
+    new, ctx, slot = [5, 1, 2, 3], [0, 4, 7, 0], [2, 0, -1, 3]
+    T = sum(new)
+    proj = _r(g, T, col0 + C + 5, dt=dt)
+    cw, cb = _r(g, C, taps, s=0.5), _r(g, C, s=0.1)
+    state = _r(g, 4, max(1, taps - 1), C, dt=dt)
+    cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
+    s_c, s_g = state.clone(), state.clone().cuda()
+    want = H.conv_silu(proj, col0, C, cw, cb, s_c, cu, _i32(ctx), _i32(slot))
+    got = H.conv_silu(proj.cuda(), col0, C, cw.cuda(), cb.cuda(), s_g, cu.cuda(), _i32(ctx).cuda(), _i32(slot).cuda())
+    live = torch.tensor([r for s in range(4) if slot[s] >= 0 for r in range(int(cu[s]), int(cu[s + 1]))])
+    torch.testing.assert_close(got.cpu().float()[live], want.float()[live], **_tol(dt))
+    if taps > 1:
+        torch.testing.assert_close(s_g.cpu().float(), s_c.float(), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("nh,P,N,G", [(4, 24, 12, 2), (2, 80, 40, 1), (3, 16, 130, 3)])
+def test_ssm_scan_with_state(dt, nh, P, N, G):
+    g = _g(6)
+    new, ctx, slot = [6, 1, 3], [0, 9, 2], [1, 3, 0]
+    T = sum(new)
+    inner = nh * P
+    xbc = _r(g, T, inner + 2 * G * N, s=0.7, dt=dt)
+    proj = _r(g, T, 11 + nh, dt=dt)
+    dtb, alog, dsk = _r(g, nh, s=0.5) - 1, _r(g, nh, s=0.5) - 0.5, _r(g, nh) + 1
+    state = _r(g, 4, nh, N, P)
+    cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
+    s_c, s_g = state.clone(), state.clone().cuda()
+    want = H.ssm_scan(xbc, proj, 11, dtb, alog, dsk, s_c, cu, _i32(ctx), _i32(slot), nh, P, N, G)
+    got = H.ssm_scan(xbc.cuda(), proj.cuda(), 11, dtb.cuda(), alog.cuda(), dsk.cuda(), s_g, cu.cuda(), _i32(ctx).cuda(),
+                     _i32(slot).cuda(), nh, P, N, G)
+    torch.testing.assert_close(got.cpu(), want, rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(s_g.cpu(), s_c, rtol=2e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("E,K,shared", [(5, 2, True), (24, 4, False), (70, 1, True)])
+def test_router_and_experts(dt, E, K, shared):
+    g = _g(7)
+    T, d, ff = 45, 72, 40
+    h = _r(g, T, d, dt=dt)
+    wr, bias = _r(g, E + (1 if shared else 0), d, s=0.3), _r(g, E, s=0.3)
+    ids_c, w_c, gate_c = H.moe_router(h, wr, bias, E, K)
+    ids_g, w_g, gate_g = H.moe_router(h.cuda(), wr.cuda(), bias.cuda(), E, K)
+    assert torch.equal(ids_g.cpu(), ids_c)
+    torch.testing.assert_close(w_g.cpu(), w_c, rtol=1e-4, atol=1e-5)
+    if shared:
+        torch.testing.assert_close(gate_g.cpu(), gate_c, rtol=1e-4, atol=1e-5)
+    w13, w2 = _r(g, E, 2 * ff, d, s=1 / math.sqrt(d), dt=dt), _r(g, E, d, ff, s=1 / math.sqrt(ff), dt=dt)
+    sh = _r(g, T, d, dt=dt) if shared else None
+    want = H.moe_experts(h, ids_c, w_c, w13, w2, sh, gate_c)
+    got = H.moe_experts(h.cuda(), ids_g, w_g, w13.cuda(), w2.cuda(), sh.cuda() if shared else None, gate_g)
+    torch.testing.assert_close(got.cpu(), want, **_tol(dt))
