@@ -201,13 +201,16 @@ def conv_silu(proj: torch.Tensor, col0: int, C: int, conv_w: torch.Tensor, conv_
             if slot < 0 or b <= a:
                 continue
             x = proj[a:b, col0:col0 + C]
-            hist = conv_state[slot] if c0 > 0 else torch.zeros_like(conv_state[slot])
+            hist = conv_state[slot, : taps - 1]
+            if c0 <= 0:
+                hist = torch.zeros_like(hist)
             full = torch.cat([hist.to(proj.dtype), x]).float()  # [taps - 1 + n, C]
             acc = bf.expand(b - a, C).clone()
             for j in range(taps):
                 acc += full[j:j + b - a] * wt[j]
             out[a:b] = _silu(acc).to(proj.dtype)
-            conv_state[slot] = full[full.shape[0] - (taps - 1):].to(conv_state.dtype)
+            if taps > 1:
+                conv_state[slot] = full[full.shape[0] - (taps - 1):].to(conv_state.dtype)
         return out
     out = torch.empty(T, C, dtype=proj.dtype, device=proj.device)
     native().conv_silu(out, proj, int(col0), conv_w, conv_b, conv_state, seg_cu, seg_ctx, seg_slot)
