@@ -17,6 +17,8 @@ Modes (``--mode``):
   at ``--rate`` queries/s; reports TTFT / TPOT / latency percentiles (mixed prefill+decode steps
   at work).
 * ``latency`` - batch 1: one query at a time; a step = one query.
+* ``arch`` - not the headline: prefill and decode tokens/s of the Dunesun layer-list design beside
+  a Mixtral-style model of equal layer sizes (engine/arch_bench.py), one GPU, random weights.
 ``--production``: the server runs with the reference's timeouts (15 s write, 30 s llm.timeout)
 instead of the bench's 600 s; answers that reach the deadline come back truncated
 (finish_reason "deadline") and overload as 503 - both are counted in the JSON line.
@@ -61,7 +63,12 @@ def parse(argv=None):
     ap.add_argument("--model", default="llama-3-8b")
     ap.add_argument("--batch", type=int, default=64, help="concurrent queries per replica per step")
     ap.add_argument("--max-new-tokens", type=int, default=256)
-    ap.add_argument("--mode", choices=["wave", "poisson", "latency"], default="wave")
+    ap.add_argument("--mode", choices=["wave", "poisson", "latency", "arch"], default="wave")
+    ap.add_argument("--arch-sizes", default="s,m", help="arch: layer sizes to compare (engine/arch_bench.py SIZES)")
+    ap.add_argument("--arch-prompt", type=int, default=2048, help="arch: prompt tokens per sequence")
+    ap.add_argument("--arch-seqs", type=int, default=4, help="arch: prompts in the prefill step")
+    ap.add_argument("--arch-window", type=int, default=1024, help="arch: the Dunesun attention layers' window")
+    ap.add_argument("--arch-which", choices=["both", "new", "ref"], default="both")
     ap.add_argument("--rate", type=float, default=16.0, help="poisson: arrivals per second per replica")
     ap.add_argument("--production", action="store_true",
                     help="reference server timeouts (15 s write / 30 s llm): deadline truncation + 503s")
@@ -490,6 +497,11 @@ def _print_trace(trace: list, t0: float) -> None:
 def main(argv=None) -> None:
     argv = list(sys.argv[1:] if argv is None else argv)
     a = parse(argv)
+    if a.mode == "arch":
+        from k8s_llm_monitor_amd.engine import arch_bench
+
+        arch_bench.run(a)
+        return
     if a.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(spawn_ranks(a.gpus, argv))
     run_rank(a)

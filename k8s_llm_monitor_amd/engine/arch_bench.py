@@ -1,0 +1,122 @@
+"""Prefill and decode throughput of the Dunesun design beside the closest existing model
+(Mixtral-style: attention + routed experts in every layer) at equal layer sizes, random weights,
+one GPU (``python bench.py --mode arch``).  Both models run through the same ModelRunner step
+functions the engine uses: one prefill step of ``seqs`` whole prompts, then decode steps of
+``batch`` sequences (hipGraph replay where the model's decode is captured)."""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+from ..models.config import HybridConfig, LayerSpec, ModelConfig, MoESpec
+from ..models.registry import build_model
+from .block_manager import BlockManager
+from .runner import ModelRunner, RunnerConfig
+from .sequence import SamplingParams, Sequence
+
+# (name, width, heads, kv heads, head dim, experts, top, expert ff, layers)
+SIZES = {
+    "s": ("d1024", 1024, 8, 2, 128, 8, 2, 1024, 4),
+    "m": ("d2048", 2048, 16, 4, 128, 8, 2, 2048, 4),
+    "l": ("d4096", 4096, 32, 8, 128, 8, 2, 3584, 2),
+}
+
+
+def _pair(size: str, window: int) -> tuple:
+    name, d, H, G, D, E, K, ff, L = SIZES[size]
+    att = LayerSpec("attention", tuple(sorted({"heads": H, "kv_heads": G, "dim": D, "vdim": D, "mask.size": window,
+                                               "scale": D ** -0.5}.items())), MoESpec(E, K, ff, 0))
+    ssm = LayerSpec("mamba2", tuple(sorted({"heads": 2 * d // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4,
+                                            "norm_groups": 1}.items())), MoESpec(E, K, ff, 0))
+    hy = HybridConfig(name=f"dunesun-{name}", arch="dunesun", vocab_size=32000, d_model=d,
+                      layers=tuple(att if i % 2 == 0 else ssm for i in range(L)), max_position=8192)
+    ref = ModelConfig(name=f"mixtral-{name}", arch="llama", vocab_size=32000, d_model=d, n_layers=L, n_heads=H,
+                      n_kv_heads=G, head_dim=D, ffn_dim=ff, max_position=8192, rope_theta=1e6, n_experts=E,
+                      top_k_experts=K, bos_id=1, eos_ids=(2,))
+    return hy, ref
+
+
+def _measure(cfg, seqs: int, prompt: int, batch: int, steps: int, warmup: int, graphs: bool) -> dict:
+    dev = torch.device("cuda:0")
+    model = build_model(cfg, device=dev, dtype=torch.bfloat16)
+    nseq = max(seqs, batch)
+    nb = nseq * ((prompt + steps + warmup + 64) // 16 + 2)
+    runner = ModelRunner(model, RunnerConfig(max_num_seqs=nseq, max_model_len=prompt + 256, num_blocks=nb,
+                                             use_graphs=graphs))
+    blocks = BlockManager(nb, prefix_caching=False, state_slots=runner.num_state_slots)
+    g = torch.Generator().manual_seed(0)
+    par = SamplingParams(temperature=0.0, ignore_eos=True)
+
+    def fresh(n):
+        qs = [Sequence(prompt_ids=torch.randint(3, 30000, (prompt,), generator=g).tolist(), params=par) for _ in range(n)]
+        for q in qs:
+            assert blocks.allocate(q)
+            q.chunk = prompt
+        return qs
+
+    def timed(fn, k):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(k):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / k
+
+    out = {"model": cfg.name, "params_m": round(model.num_local_params() / 1e6, 1)}
+    with torch.no_grad():
+        qs = fresh(seqs)
+
+        def pf():
+            for q in qs:
+                q.num_computed = 0
+            runner.prefill(qs)
+
+        timed(pf, warmup)
+        t = timed(pf, steps)
+        out["prefill_ms"] = round(t * 1e3, 3)
+        out["prefill_tok_s"] = round(seqs * prompt / t, 1)
+        for q in qs:
+            blocks.free(q)
+        qs = fresh(batch)
+        toks = runner.prefill(qs)
+        for q, tk in zip(qs, toks):
+            q.num_computed, q.chunk, q.prefilled = prompt, 0, True
+            q.output_ids.append(int(tk))
+        if graphs:
+            runner.capture_graphs([runner.bucket_for(batch)])
+
+        def dec():
+            for q in qs:
+                assert blocks.ensure_slot(q)
+            for q, tk in zip(qs, runner.decode(qs)):
+                q.output_ids.append(int(tk))
+
+        timed(dec, warmup)
+        t = timed(dec, steps)
+        out["decode_ms"] = round(t * 1e3, 3)
+        out["decode_tok_s"] = round(batch / t, 1)
+    del runner, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def run(a) -> None:
+    """``a``: bench.py's parsed arguments (arch_sizes, arch_prompt, arch_seqs, batch, steps, warmup)."""
+    rows = []
+    for size in a.arch_sizes.split(","):
+        hy, ref = _pair(size, a.arch_window)
+        for cfg in ((hy, ref) if a.arch_which == "both" else ((hy,) if a.arch_which == "new" else (ref,))):
+            r = _measure(cfg, a.arch_seqs, a.arch_prompt, a.batch, a.steps, a.warmup, not a.no_graphs)
+            r["size"] = size
+            rows.append(r)
+            print(json.dumps(r), flush=True)
+    line = {"metric": "arch_compare_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "dtype": "bf16", "data": "synthetic", "higher_is_better": True,
+            "config": {"prompt": a.arch_prompt, "prefill_seqs": a.arch_seqs, "decode_batch": a.batch,
+                       "window": a.arch_window}, "rows": rows}
+    print(json.dumps(line), flush=True)
+    if a.out:
+        with open(a.out, "w") as f:
+            f.write(json.dumps(line) + "\n")
