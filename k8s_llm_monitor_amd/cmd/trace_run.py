@@ -55,6 +55,10 @@ def main(argv=None) -> int:
     eng = LLMEngine(EngineConfig(model=a.model, weights=a.model, dtype=a.dtype, max_num_seqs=MAX_SEQS,
                                  max_model_len=1 << 30, num_blocks=nb, use_graphs=a.graphs, keep_logits=True,
                                  prefix_caching=False, pipeline=False), device=dev)
+    if getattr(eng.model, "uses_tile_gemm", False) and dev != "cpu":
+        from ..ops import build
+
+        build.ensure(("ops",))  # large steps of this model's experts run on the prefill tile GEMM
     if a.graphs:
         eng.warmup()
     runner, blocks = eng.runner, eng.blocks

@@ -25,6 +25,7 @@ from typing import Optional
 import torch
 import torch.nn.functional as F
 
+from .. import ops as _ops
 from ..ops import hybrid as hops
 from ..parallel.state import ParallelState, get_state
 from .config import HybridConfig, LayerSpec, MoESpec
@@ -165,8 +166,12 @@ class RoutedFFN:
         if not 1 <= self.K <= self.E:
             raise ValueError(f"{prefix}: top {self.K} of {self.E} experts")
         s, s2 = 1.0 / math.sqrt(d), 1.0 / math.sqrt(self.ff)
-        self.w13 = torch.stack([torch.cat([p.get(f"{prefix}e{e}.gate", (self.ff, d), s),
-                                           p.get(f"{prefix}e{e}.up", (self.ff, d), s)]) for e in range(self.E)])
+        # gate / up rows interleaved per 128 ([64 gate | 64 up]): the layout of the prefill tile GEMM's
+        # SwiGLU epilogue, which large bf16 steps on the GPU use (ops.hybrid.moe_experts); ONE copy
+        self.il = (p.device.type == "cuda" and p.dtype == torch.bfloat16 and self.ff % 128 == 0 and d % 128 == 0)
+        pair = _ops.interleave_gate_up if self.il else (lambda w: w)
+        self.w13 = torch.stack([pair(torch.cat([p.get(f"{prefix}e{e}.gate", (self.ff, d), s),
+                                                p.get(f"{prefix}e{e}.up", (self.ff, d), s)])) for e in range(self.E)])
         self.w2 = torch.stack([p.get(f"{prefix}e{e}.down", (d, self.ff), s2) for e in range(self.E)])
         wr = p.get(prefix + "router", (self.E, d), 2 * s, small=True)
         self.bias = p.get(prefix + "router.b", (self.E,), 0.2, small=True)
@@ -183,7 +188,7 @@ class RoutedFFN:
         shared = None
         if self.fs:
             shared = F.linear(hops.swiglu(F.linear(h, self.ws13)), self.ws2)
-        return hops.moe_experts(h, ids, wts, self.w13, self.w2, shared, gate)
+        return hops.moe_experts(h, ids, wts, self.w13, self.w2, shared, gate, il=self.il)
 
 
 class HybridLM:
@@ -219,6 +224,8 @@ class HybridLM:
         self.runs = cfg.runs()
         self.unused = sorted(set(weights.keys()) - p.used) if weights is not None else []
         self.has_state = any(m.kind != "attention" for m in self.mixers)
+        # large steps of such layers run on the Mixtral path's tile GEMM (extension _k8sllm_ops)
+        self.uses_tile_gemm = any(f is not None and f.il for f in self.ffns)
         self.layer_probe = None  # a list: forward() appends the residual stream after every run
 
     # ------------------------------------------------------------------ engine interface
@@ -297,7 +304,8 @@ def state_dict(model: HybridLM) -> dict:
                         p + "mix.norm": m.norm_w, p + "mix.o": m.wo})
         if f is not None:
             for e in range(f.E):
-                out[f"{p}mlp.e{e}.gate"], out[f"{p}mlp.e{e}.up"] = f.w13[e, :f.ff], f.w13[e, f.ff:]
+                w13 = _ops.deinterleave_gate_up(f.w13[e]) if f.il else f.w13[e]
+                out[f"{p}mlp.e{e}.gate"], out[f"{p}mlp.e{e}.up"] = w13[:f.ff], w13[f.ff:]
                 out[f"{p}mlp.e{e}.down"] = f.w2[e]
             out[p + "mlp.router"], out[p + "mlp.router.b"] = f.wr[:f.E], f.bias
             if f.fs:

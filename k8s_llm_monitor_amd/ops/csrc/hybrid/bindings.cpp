@@ -19,10 +19,10 @@ int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float
 int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                              const int* cu, const int* ctx, const int* block_tables, int bt_stride, int S, long T,
                              int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink, int f32,
-                             hipStream_t s);
+                             int mfma, hipStream_t s);
 int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                             const int* block_tables, int bt_stride, const int* seq_lens, int B, int Hq, int G, int dk,
-                            int dv, int bs, float scale, int window, int sink, int f32, hipStream_t s);
+                            int dv, int bs, float scale, int window, int sink, int f32, int vec, hipStream_t s);
 int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int C, const float* cw, const float* cb,
                         int taps, void* state, const int* cu, const int* ctx, const int* slot, int S, long T, int f32,
                         hipStream_t s);
@@ -32,7 +32,8 @@ int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_strid
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
                      const float* bias, int E, int K, int rows_w, int f32, hipStream_t s);
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
-                           int E, long rows, int N, int Kd, long w_es, int swiglu, int f32, hipStream_t s);
+                           int E, long rows, int N, int Kd, long w_es, int swiglu, int il, int f32, int mfma,
+                           hipStream_t s);
 int k8sllm_hy_combine(float* out, const void* ys, const int* inv, const float* wts, const void* shared,
                       const float* gate, long T, int K, int d, int f32, hipStream_t s);
 int k8sllm_moe_align(const int* topk_ids, long n, int E, int* expert_offsets, int* sorted_idx, int* inv_idx,
@@ -174,7 +175,7 @@ void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int
 
 void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor cu, Tensor ctx,
                               Tensor block_tables, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
-                              int64_t window, bool sink) {
+                              int64_t window, bool sink, bool mfma) {
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
@@ -192,13 +193,13 @@ void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_c
   check(k8sllm_hy_window_prefill(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  cu.data_ptr<int>(), ctx.data_ptr<int>(), block_tables.data_ptr<int>(),
                                  (int)block_tables.stride(0), (int)S, T, (int)Hq, (int)G, (int)dk, (int)dv,
-                                 (int)k_cache.size(1), (float)scale, (int)window, sink, f, cur()),
+                                 (int)k_cache.size(1), (float)scale, (int)window, sink, f, mfma, cur()),
         "window_attention_prefill");
 }
 
 void window_attention_decode(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor block_tables,
                              Tensor seq_lens, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
-                             int64_t window, bool sink) {
+                             int64_t window, bool sink, bool vec) {
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
@@ -215,7 +216,7 @@ void window_attention_decode(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_ca
   check(k8sllm_hy_window_decode(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                 block_tables.data_ptr<int>(), (int)block_tables.stride(0), seq_lens.data_ptr<int>(),
                                 (int)B, (int)Hq, (int)G, (int)dk, (int)dv, (int)k_cache.size(1), (float)scale,
-                                (int)window, sink, f, cur()),
+                                (int)window, sink, f, vec, cur()),
         "window_attention_decode");
 }
 
@@ -305,7 +306,8 @@ void moe_align(Tensor ids, int64_t E, Tensor offsets, Tensor sorted_idx, Tensor 
 }
 
 // y [rows, N] = W[e] a over expert-sorted rows; sorted_idx given: a's row of sorted row r is sorted_idx[r] / div
-void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx, int64_t div, bool swiglu) {
+void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx, int64_t div, bool swiglu, bool il,
+                  bool mfma) {
   const int f = act(a, "a");
   same(y, f, "y");
   same(w, f, "w");
@@ -316,6 +318,7 @@ void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx,
   const int64_t N = swiglu ? w.size(1) / 2 : w.size(1);
   TORCH_CHECK(a.size(1) == Kd && y.size(1) == N && offsets.numel() == E + 1 && (!swiglu || w.size(1) % 2 == 0),
               "grouped_gemm: shapes");
+  TORCH_CHECK(!il || (swiglu && N % 64 == 0), "grouped_gemm: interleaved gate/up needs swiglu and ff % 64 == 0");
   const int* sp = iptr(sorted_idx, "sorted_idx");
   if (sp) {
     TORCH_CHECK(sorted_idx->numel() == rows && div >= 1 && a.size(0) * div >= rows, "grouped_gemm: gather index");
@@ -323,7 +326,7 @@ void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx,
     TORCH_CHECK(a.size(0) == rows, "grouped_gemm: a rows");
   }
   check(k8sllm_hy_grouped_gemm(y.data_ptr(), a.data_ptr(), w.data_ptr(), offsets.data_ptr<int>(), sp, (int)div, (int)E,
-                               rows, (int)N, (int)Kd, w.size(1) * Kd, swiglu, f, cur()),
+                               rows, (int)N, (int)Kd, w.size(1) * Kd, swiglu, il, f, mfma, cur()),
         "grouped_gemm");
 }
 

@@ -68,7 +68,7 @@ template <typename T, bool SWIGLU>
 __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y, const T* __restrict__ A,
                                                               const T* __restrict__ W, const int* __restrict__ offsets,
                                                               const int* __restrict__ sorted_idx, int div, int E,
-                                                              int N, int Kd, long w_es) {
+                                                              int N, int Kd, long w_es, int il) {
   __shared__ float As[TK][TM + 4];
   __shared__ float Ws[TK][TN + 4];
   __shared__ float Us[SWIGLU ? TK : 1][TN + 4];
@@ -98,13 +98,16 @@ __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y,
   long asrc = -1;
   if (arow < r1) asrc = sorted_idx != nullptr ? sorted_idx[arow] / div : arow;
   const int wrow = n0 + lr;
+  // row of W holding output column wrow's gate (or only) weights, and its up weights
+  const long grow = SWIGLU && il ? (long)(wrow >> 6) * 128 + (wrow & 63) : wrow;
+  const long urow = il ? grow + 64 : (long)N + wrow;
   for (int k0 = 0; k0 < Kd; k0 += TK) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = k0 + lk + j;
       As[lk + j][lr] = (asrc >= 0 && k < Kd) ? ldf(A + asrc * Kd + k) : 0.f;
-      Ws[lk + j][lr] = (wrow < N && k < Kd) ? ldf(We + (long)wrow * Kd + k) : 0.f;
-      if (SWIGLU) Us[lk + j][lr] = (wrow < N && k < Kd) ? ldf(We + (long)(N + wrow) * Kd + k) : 0.f;
+      Ws[lk + j][lr] = (wrow < N && k < Kd) ? ldf(We + grow * Kd + k) : 0.f;
+      if (SWIGLU) Us[lk + j][lr] = (wrow < N && k < Kd) ? ldf(We + urow * Kd + k) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -149,6 +152,71 @@ __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y,
   }
 }
 
+// bf16 on the matrix cores (K a multiple of 32): one wave = 16 sorted rows x 64 output columns,
+// v_mfma_f32_16x16x32_bf16 with both operands loaded straight from global memory as 16-byte
+// fragments (A = the gathered activation rows, B = weight rows, 8 consecutive k per lane).  Few
+// rows per expert (decode) make this a weight-streaming kernel: many small workgroups, no LDS.
+// ``il``: the gate / up rows are interleaved per 128 rows as [64 gate | 64 up] (the prefill tile
+// GEMM's pairing), else [all gate rows ; all up rows].
+template <bool SWIGLU>
+__global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __restrict__ Y, const bf16_t* __restrict__ A,
+                                                                  const bf16_t* __restrict__ W,
+                                                                  const int* __restrict__ offsets,
+                                                                  const int* __restrict__ sorted_idx, int div, int E,
+                                                                  int N, int Kd, long w_es, int il) {
+  int e = 0, tile = blockIdx.x, r0 = 0, r1 = 0;
+  for (; e < E; ++e) {
+    r0 = offsets[e];
+    r1 = offsets[e + 1];
+    const int nt = (r1 - r0 + 15) >> 4;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (e >= E) return;
+  r0 += tile * 16;
+  const int lane = threadIdx.x, c16 = lane & 15, quad = lane >> 4;
+  const int n0 = blockIdx.y * 64;
+  const bf16_t* We = W + (long)e * w_es;
+  const int arow = min(r0 + c16, r1 - 1);
+  const long asrc = sorted_idx != nullptr ? sorted_idx[arow] / div : arow;
+  const bf16_t* ap = A + asrc * Kd + 8 * quad;
+  const bf16_t* wg[4];
+  const bf16_t* wu[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int n = min(n0 + 16 * t + c16, N - 1);
+    const long g = SWIGLU && il ? (long)(n >> 6) * 128 + (n & 63) : n;
+    wg[t] = We + g * Kd + 8 * quad;
+    wu[t] = We + (SWIGLU ? (il ? g + 64 : (long)N + n) : 0) * Kd + 8 * quad;
+  }
+  f32x4 acc[4], accu[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) acc[t] = accu[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k0 = 0; k0 < Kd; k0 += 32) {
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(ap + k0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, *reinterpret_cast<const bf16x8*>(wg[t] + k0), acc[t], 0, 0, 0);
+      if (SWIGLU)
+        accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, *reinterpret_cast<const bf16x8*>(wu[t] + k0), accu[t], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {  // acc[t][i]: row r0 + 4 quad + i, column n0 + 16 t + c16
+    const int n = n0 + 16 * t + c16;
+    if (n >= N) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = r0 + 4 * quad + i;
+      if (r >= r1) continue;
+      float v = acc[t][i];
+      if (SWIGLU) v = silu_f(bf2f(f2bf(v))) * bf2f(f2bf(accu[t][i]));
+      Y[(long)r * N + n] = f2bf(v);
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void hy_combine_kernel(float* __restrict__ out, const T* __restrict__ ys,
                                                          const int* __restrict__ inv, const float* __restrict__ wts,
@@ -184,12 +252,24 @@ int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, i
 
 // rows: the sorted rows in all (an upper bound of the row tiles is rows / 64 + E)
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
-                           int E, long rows, int N, int Kd, long w_es, int swiglu, int f32, hipStream_t s) {
+                           int E, long rows, int N, int Kd, long w_es, int swiglu, int il, int f32, int mfma,
+                           hipStream_t s) {
   if (rows <= 0) return 0;
+  if (il && (!swiglu || N % 64)) return -1;
+  if (!f32 && mfma && Kd % 32 == 0) {
+    const dim3 g16((unsigned)(rows / 16 + E), (unsigned)((N + 63) / 64));
+    if (swiglu)
+      hipLaunchKernelGGL(hy_grouped_gemm_mfma_kernel<true>, g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,
+                         (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il);
+    else
+      hipLaunchKernelGGL(hy_grouped_gemm_mfma_kernel<false>, g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,
+                         (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il);
+    return (int)hipGetLastError();
+  }
   const dim3 grid((unsigned)(rows / TM + E), (unsigned)((N + TN - 1) / TN));
 #define K8SLLM_GG(T, SW)                                                                                            \
   hipLaunchKernelGGL((hy_grouped_gemm_kernel<T, SW>), grid, dim3(256), 0, s, (T*)Y, (const T*)A, (const T*)W, offsets, \
-                     sorted_idx, div, E, N, Kd, w_es)
+                     sorted_idx, div, E, N, Kd, w_es, il)
   if (f32) {
     if (swiglu) K8SLLM_GG(float, true); else K8SLLM_GG(float, false);
   } else {

@@ -135,6 +135,216 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
                  n, h / (Hq / G), G, dk, dv, bs, scale, sink, q_s, p_s);
 }
 
+// bf16 decode with 16-byte loads: one wave per (sequence, kv head) serves all R = Hq / G query
+// heads of that kv head, so every cached key and value row is read once.  Scores: lane = key, the
+// lane walks its key row in 8-element pieces against the R queries held in LDS (fp32).  Values:
+// lane = (key subset, 8-dim piece); each lane accumulates its piece over its subset's keys and the
+// subsets meet through xor-shuffles once at the end.  Needs dk % 8 == 0 and dv / 8 a power of two.
+template <int R>
+__global__ __launch_bounds__(64) void window_decode_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv,
+                                                               long q_stride, const bf16_t* __restrict__ k_cache,
+                                                               const bf16_t* __restrict__ v_cache,
+                                                               const int* __restrict__ block_tables, int bt_stride,
+                                                               const int* __restrict__ seq_lens, int Hq, int G, int dk,
+                                                               int dv, int bs, float scale, int window, int sink) {
+  __shared__ __attribute__((aligned(16))) float q_s[R * kMaxDK];
+  __shared__ float p_s[R][64];
+  const int b = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  const int n = seq_lens[b];
+  const int DL = dv >> 3;            // lanes that cover the value dims, 8 each
+  const int dg = lane & (DL - 1), ksub = lane / DL, KS = 64 / DL;
+  bf16_t* o = out + (long)b * Hq * dv + (long)g * R * dv;
+  if (n <= 0) {  // padding row of a decode bucket
+    for (int c = lane; c < R * dv; c += 64) o[c] = 0;
+    return;
+  }
+  const bf16_t* q = qkv + (long)b * q_stride + (long)g * R * dk;
+  for (int c = lane; c < R * dk; c += 64) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * scale;
+  __syncthreads();
+  const int* bt = block_tables + (long)b * bt_stride;
+  const int lo = window > 0 ? max(0, n - window) : 0;
+  float m[R], l[R], acc[R][8];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    m[r] = sink ? 0.f : -INFINITY;
+    l[r] = sink ? 1.f : 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
+  }
+  const long krs = (long)G * dk, vrs = (long)G * dv;
+  for (int j0 = lo; j0 < n; j0 += 64) {
+    const int j = j0 + lane;
+    float sc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) sc[r] = 0.f;
+    if (j < n) {
+      const bf16_t* kp = k_cache + ((long)bt[j / bs] * bs + j % bs) * krs + (long)g * dk;
+      for (int c = 0; c < dk; c += 8) {
+        float kv[8];
+        unpack8(*reinterpret_cast<const uint4*>(kp + c), kv);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float4 qa = *reinterpret_cast<const float4*>(&q_s[r * kMaxDK + c]);
+          const float4 qb = *reinterpret_cast<const float4*>(&q_s[r * kMaxDK + c + 4]);
+          sc[r] += kv[0] * qa.x + kv[1] * qa.y + kv[2] * qa.z + kv[3] * qa.w + kv[4] * qb.x + kv[5] * qb.y +
+                   kv[6] * qb.z + kv[7] * qb.w;
+        }
+      }
+    }
+    __syncthreads();  // the previous tile's reads of p_s are done
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float s = j < n ? sc[r] : -INFINITY;
+      const float mt = fmaxf(m[r], wave_max(s));
+      const float p = j < n ? expf(s - mt) : 0.f;
+      const float alpha = m[r] == -INFINITY ? 0.f : expf(m[r] - mt);
+      l[r] = l[r] * alpha + wave_sum(p);
+      m[r] = mt;
+      p_s[r][lane] = p;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[r][i] *= alpha;
+    }
+    __syncthreads();
+    const int cnt = min(64, n - j0);
+    for (int i = ksub; i < cnt; i += KS) {
+      const int jj = j0 + i;
+      float vv[8];
+      unpack8(*reinterpret_cast<const uint4*>(v_cache + ((long)bt[jj / bs] * bs + jj % bs) * vrs + (long)g * dv + dg * 8),
+              vv);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float p = p_s[r][i];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[r][k] += p * vv[k];
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float a = acc[r][k];
+      for (int off = DL; off < 64; off <<= 1) a += __shfl_xor(a, off, 64);
+      acc[r][k] = a;
+    }
+    if (ksub == 0) {
+      const float inv = l[r] > 0.f ? 1.f / l[r] : 0.f;
+      float w[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) w[k] = acc[r][k] * inv;
+      *reinterpret_cast<uint4*>(o + (long)r * dv + dg * 8) = pack8(w);
+    }
+  }
+}
+
+// bf16 prefill on the matrix cores, head sizes that are multiples of 32 (keys) / 16 (values).
+// One wave = 16 consecutive chunk rows of one sequence x one query head; key tiles of 16.
+//   S^T[key][q]  = K Q^T      v_mfma_f32_16x16x32_bf16: A = K rows (16-byte loads straight from the
+//                             pages), B = the wave's Q rows (held in registers for the whole loop)
+//   O^T[d][q]   += V^T P^T    v_mfma_f32_16x16x16_bf16: B = the score accumulator itself (query on
+//                             the lane, 4 keys per lane: the C layout of S^T IS the B layout of P^T),
+//                             A = V^T read back transposed from an LDS copy of the 16-key V tile
+// With the query on the lane the running maximum, denominator and the rescale of O are lane-local
+// (two xor-shuffles per reduction).  Scores, weights and sums are fp32; P is rounded to bf16 for
+// the PV product.
+template <int DK, int DV>
+__global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv, long q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
+    const int* __restrict__ block_tables, int bt_stride, int S, int Hq, int G, int bs, float scale, int window,
+    int sink) {
+  constexpr int VP = DV + 16;  // LDS row pitch: the 4 key rows of a fragment read land 8 banks apart
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * VP];
+  int tile = blockIdx.x, s = 0, n = 0;
+  for (; s < S; ++s) {  // q-tiles are numbered segment by segment
+    n = cu[s + 1] - cu[s];
+    const int nt = (n + 15) >> 4;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= S) return;
+  const int q0 = tile * 16, nq = min(16, n - q0);
+  const int h = blockIdx.y, g = h / (Hq / G);
+  const int lane = threadIdx.x, c16 = lane & 15, quad = lane >> 4;
+  const int* bt = block_tables + (long)s * bt_stride;
+  const int row0 = cu[s] + q0, p0 = ctx[s] + q0;
+  const int myq = min(c16, nq - 1);
+  const int my_p = p0 + myq;
+  const int my_lo = window > 0 ? max(0, my_p - window + 1) : 0;
+  const bool q_live = c16 < nq;
+  bf16x8 qf[DK / 32];
+  const bf16_t* qrow = qkv + (long)(row0 + myq) * q_stride + (long)h * DK;
+#pragma unroll
+  for (int ks = 0; ks < DK / 32; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * quad);
+  f32x4 oacc[DV / 16];
+#pragma unroll
+  for (int dt = 0; dt < DV / 16; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  const int lo_t = window > 0 ? max(0, p0 - window + 1) : 0, hi = p0 + nq;
+  const long krs = (long)G * DK, vrs = (long)G * DV;
+  for (int j0 = lo_t & ~15; j0 < hi; j0 += 16) {
+    const int jk = min(j0 + c16, hi - 1);
+    const bf16_t* krow = k_cache + ((long)bt[jk / bs] * bs + jk % bs) * krs + (long)g * DK;
+    f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < DK / 32; ++ks)
+      sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + 32 * ks + 8 * quad),
+                                                     qf[ks], sacc, 0, 0, 0);
+    float sv[4], tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, query c16
+      const int j = j0 + 4 * quad + i;
+      sv[i] = (q_live && j >= my_lo && j <= my_p) ? sacc[i] * scale : -INFINITY;
+      tmax = fmaxf(tmax, sv[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);
+    const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
+    float pv[4], ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pv[i] = sv[i] == -INFINITY ? 0.f : expf(sv[i] - mn);
+      ps += pv[i];
+    }
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * alpha + ps;
+    m = mn;
+    s16x4 pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pb[i] = (short)f2bf(pv[i]);
+    __syncthreads();  // one wave per workgroup: the previous tile's fragment reads are done
+    for (int c = lane; c < 16 * (DV / 8); c += 64) {
+      const int key = c / (DV / 8), dc = c % (DV / 8);
+      const int jv = min(j0 + key, hi - 1);
+      const bf16_t* vrow = v_cache + ((long)bt[jv / bs] * bs + jv % bs) * vrs + (long)g * DV;
+      *reinterpret_cast<uint4*>(&Vs[key * VP + dc * 8]) = *reinterpret_cast<const uint4*>(vrow + dc * 8);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int dt = 0; dt < DV / 16; ++dt) {
+      s16x4 a;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = (short)Vs[(4 * quad + i) * VP + 16 * dt + c16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
+      oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dt], 0, 0, 0);
+    }
+  }
+  if (q_live) {  // oacc[dt][i] = O[q = c16][d = 16 dt + 4 quad + i]
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* orow = out + (long)(row0 + c16) * Hq * DV + (long)h * DV;
+#pragma unroll
+    for (int dt = 0; dt < DV / 16; ++dt) {
+      uint2 w;
+      w.x = pack2(oacc[dt][0] * inv, oacc[dt][1] * inv);
+      w.y = pack2(oacc[dt][2] * inv, oacc[dt][3] * inv);
+      *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * quad) = w;
+    }
+  }
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -156,9 +366,23 @@ int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float
 int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                              const int* cu, const int* ctx, const int* block_tables, int bt_stride, int S, long T,
                              int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink, int f32,
-                             hipStream_t s) {
+                             int mfma, hipStream_t s) {
   if (T <= 0 || S <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
+  // bf16 with matrix-core head sizes and 16-byte aligned rows: the MFMA kernel
+  if (!f32 && mfma && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
+    const dim3 grid((unsigned)(T / 16 + S), (unsigned)Hq);
+#define K8SLLM_WP(DK, DV)                                                                                             \
+  hipLaunchKernelGGL((window_prefill_mfma_kernel<DK, DV>), grid, dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,      \
+                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, block_tables, bt_stride, S, Hq, \
+                     G, bs, scale, window, sink)
+    if (dk == 64 && dv == 64) K8SLLM_WP(64, 64);
+    else if (dk == 64) K8SLLM_WP(64, 128);
+    else if (dv == 64) K8SLLM_WP(128, 64);
+    else K8SLLM_WP(128, 128);
+#undef K8SLLM_WP
+    return (int)hipGetLastError();
+  }
   if (f32)
     hipLaunchKernelGGL(window_prefill_kernel<float>, dim3(T, Hq), dim3(64), 0, s, (float*)out, (const float*)qkv,
                        q_stride, (const float*)k_cache, (const float*)v_cache, cu, ctx, block_tables, bt_stride, S, Hq,
@@ -172,9 +396,23 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
 
 int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                             const int* block_tables, int bt_stride, const int* seq_lens, int B, int Hq, int G, int dk,
-                            int dv, int bs, float scale, int window, int sink, int f32, hipStream_t s) {
+                            int dv, int bs, float scale, int window, int sink, int f32, int vec, hipStream_t s) {
   if (B <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
+  const int R = Hq / G, DL = dv / 8;
+  if (!f32 && vec && dk % 8 == 0 && dv % 8 == 0 && DL >= 1 && DL <= 64 && (DL & (DL - 1)) == 0 && q_stride % 8 == 0 &&
+      (R == 1 || R == 2 || R == 4 || R == 8)) {
+#define K8SLLM_WD(RR)                                                                                                  \
+  hipLaunchKernelGGL(window_decode_vec_kernel<RR>, dim3(B, G), dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,          \
+                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_stride, seq_lens, Hq, G, \
+                     dk, dv, bs, scale, window, sink)
+    if (R == 1) K8SLLM_WD(1);
+    else if (R == 2) K8SLLM_WD(2);
+    else if (R == 4) K8SLLM_WD(4);
+    else K8SLLM_WD(8);
+#undef K8SLLM_WD
+    return (int)hipGetLastError();
+  }
   if (f32)
     hipLaunchKernelGGL(window_decode_kernel<float>, dim3(B, Hq), dim3(64), 0, s, (float*)out, (const float*)qkv,
                        q_stride, (const float*)k_cache, (const float*)v_cache, block_tables, bt_stride, seq_lens, Hq, G,

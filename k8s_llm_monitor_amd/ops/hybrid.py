@@ -130,11 +130,12 @@ def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, sin
 
 def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu: torch.Tensor,
                              ctx: torch.Tensor, block_tables: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int,
-                             scale: float, window: int, sink: bool) -> torch.Tensor:
+                             scale: float, window: int, sink: bool, mfma: bool = True) -> torch.Tensor:
     """Attention of the step's prompt chunks over the paged cache (which already holds their own
     keys): row r of segment s at position p = ctx[s] + r sees positions max(0, p - window + 1) .. p
     (``window`` 0: all of 0 .. p).  ``sink``: the softmax denominator has one more term exp(0) that
-    carries no value.  Scores and weights are fp32.  Returns [T, Hq*dv]."""
+    carries no value.  Scores and weights are fp32.  Returns [T, Hq*dv].  GPU, bf16, head sizes
+    64 / 128: the matrix-core kernel (``mfma=False``: the any-size wave-per-row kernel)."""
     T = qkv.shape[0]
     if not qkv.is_cuda:
         out = torch.empty(T, Hq * dv, dtype=qkv.dtype)
@@ -153,13 +154,13 @@ def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: 
         return out
     out = torch.empty(T, Hq * dv, dtype=qkv.dtype, device=qkv.device)
     native().window_attention_prefill(out, qkv, k_cache, v_cache, cu, ctx, block_tables, Hq, Hkv, dk, dv, float(scale),
-                                      int(window), bool(sink))
+                                      int(window), bool(sink), bool(mfma))
     return out
 
 
 def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             block_tables: torch.Tensor, seq_lens: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int,
-                            scale: float, window: int, sink: bool) -> torch.Tensor:
+                            scale: float, window: int, sink: bool, vec: bool = True) -> torch.Tensor:
     """One query per sequence (its newest token, already in the cache) over the last ``window``
     cached positions; ``seq_lens`` count that token (0: a padding row, output zero)."""
     B = qkv.shape[0]
@@ -177,7 +178,7 @@ def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: t
         return out
     out = torch.empty(B, Hq * dv, dtype=qkv.dtype, device=qkv.device)
     native().window_attention_decode(out, qkv, k_cache, v_cache, block_tables, seq_lens, Hq, Hkv, dk, dv, float(scale),
-                                     int(window), bool(sink))
+                                     int(window), bool(sink), bool(vec))
     return out
 
 
@@ -291,15 +292,24 @@ def moe_router(h: torch.Tensor, wr: torch.Tensor, bias: torch.Tensor, E: int, K:
     return ids, wts, gate
 
 
+# expert-sorted rows from which the routed GEMMs of an interleaved (``il``) layer go to the
+# framework's 256 x 256 prefill tile kernel (ops.moe_grouped_gemm) instead of the 16-row kernel
+TILE_MIN_ROWS = 1024
+
+
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
-                shared: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                shared: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, il: bool = False,
+                mfma: bool = True) -> torch.Tensor:
     """Sum over each token's chosen experts of ``wts * down_e(silu(gate_e h) * up_e h)`` with
-    ``w13`` [E, 2*ff, d] (gate rows then up rows) and ``w2`` [E, d, ff], plus ``gate * shared``
-    (the shared expert's output [T, d] and its per-token gate).  fp32 [T, d].
+    ``w13`` [E, 2*ff, d] (gate rows then up rows; ``il``: interleaved per 128 rows as [64 gate |
+    64 up], ops.interleave_gate_up) and ``w2`` [E, d, ff], plus ``gate * shared`` (the shared
+    expert's output [T, d] and its per-token gate).  fp32 [T, d].
 
     GPU: the (token, slot) pairs are counting-sorted by expert on the device and both projections
-    run as ONE grouped launch each over the sorted rows (gathered on load, SwiGLU in the first
-    epilogue); no host synchronisation."""
+    run as ONE grouped launch each over the sorted rows (SwiGLU in the first epilogue); no host
+    synchronisation.  bf16: matrix-core kernels - 16-row tiles with the rows gathered on load
+    (decode, small steps), or from TILE_MIN_ROWS sorted rows of an ``il`` layer the prefill tile
+    GEMM of the Mixtral path; fp32 (and K not a multiple of 32): the 64 x 64 fp32 tile kernel."""
     T, d = h.shape
     E, K = w13.shape[0], ids.shape[1]
     ff = w2.shape[2]
@@ -309,7 +319,10 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
         for e in range(E):
             rows, slot = torch.nonzero(ids == e, as_tuple=True)
             if rows.numel():
-                gu = (hf[rows] @ w13[e].float().t()).to(h.dtype).float()
+                we = w13[e].float()
+                if il:
+                    we = we.view(ff // 64, 2, 64, d).permute(1, 0, 2, 3).reshape(2 * ff, d)
+                gu = (hf[rows] @ we.t()).to(h.dtype).float()
                 act = (_silu(gu[:, :ff]) * gu[:, ff:]).to(h.dtype).float()
                 out.index_add_(0, rows, (act @ w2[e].float().t()).to(h.dtype).float() * wts[rows, slot].unsqueeze(-1))
         if shared is not None:
@@ -321,10 +334,17 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
     sorted_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     inv_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     ext.moe_align(ids, E, offsets, sorted_idx, inv_idx)
-    act = torch.empty(n, ff, dtype=h.dtype, device=h.device)
-    ext.grouped_gemm(act, h, w13, offsets, sorted_idx, K, True)
-    ys = torch.empty(n, d, dtype=h.dtype, device=h.device)
-    ext.grouped_gemm(ys, act, w2, offsets, None, 1, False)
+    if il and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16:
+        from .. import ops  # the Mixtral path's kernels (_k8sllm_ops)
+
+        xs = ops.gather_rows(h, sorted_idx, K)
+        act = ops.moe_grouped_gemm(xs, w13, offsets, swiglu=True, zero_fill=False)
+        ys = ops.moe_grouped_gemm(act, w2, offsets, zero_fill=False)
+    else:
+        act = torch.empty(n, ff, dtype=h.dtype, device=h.device)
+        ext.grouped_gemm(act, h, w13, offsets, sorted_idx, K, True, il, mfma)
+        ys = torch.empty(n, d, dtype=h.dtype, device=h.device)
+        ext.grouped_gemm(ys, act, w2, offsets, None, 1, False, False, mfma)
     out = torch.empty(T, d, dtype=torch.float32, device=h.device)
     ext.moe_combine(out, ys, inv_idx, wts, shared, gate)
     return out

@@ -168,3 +168,84 @@ def test_router_and_experts(dt, E, K, shared):
     want = H.moe_experts(h, ids_c, w_c, w13, w2, sh, gate_c)
     got = H.moe_experts(h.cuda(), ids_g, w_g, w13.cuda(), w2.cuda(), sh.cuda() if shared else None, gate_g)
     torch.testing.assert_close(got.cpu(), want, **_tol(dt))
+
+
+# ------------------------------------------------------------------ matrix-core / vector paths (bf16)
+
+@pytest.mark.parametrize("dk,dv,Hq,G", [(64, 64, 4, 2), (128, 128, 2, 1), (64, 128, 3, 3), (128, 64, 8, 2)])
+@pytest.mark.parametrize("window,sink", [(5, True), (16, True), (40, False), (0, True), (17, True)])
+def test_window_prefill_mfma(dk, dv, Hq, G, window, sink):
+    """Chunks that start inside a page, are shorter than a 16-row tile, or end one row into a tile;
+    windows at, below and above the tile size."""
+    g = _g(8)
+    dt = torch.bfloat16
+    ctx, new = [0, 40, 130, 7, 16], [37, 5, 33, 1, 16]
+    lens = [c + n for c, n in zip(ctx, new)]
+    kc, vc, bt = _paged(g, dt, lens, Hq, G, dk, dv)
+    cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
+    qkv = _r(g, sum(new), Hq * dk + G * (dk + dv), dt=dt)
+    a = (Hq, G, dk, dv, 1.0 / math.sqrt(dk), window, sink)
+    want = H.window_attention_prefill(qkv, kc, vc, cu, _i32(ctx), bt, *a)
+    dev = [t.cuda() for t in (qkv, kc, vc, cu, _i32(ctx), bt)]
+    got = H.window_attention_prefill(*dev, *a, mfma=True)
+    plain = H.window_attention_prefill(*dev, *a, mfma=False)
+    torch.testing.assert_close(plain.cpu().float(), want.float(), **_tol(dt))
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+
+
+def test_window_prefill_mfma_sees_exactly_the_window():
+    """One key with a huge value: rows whose window holds it and rows whose window has just lost it."""
+    g = _g(9)
+    dt = torch.bfloat16
+    Hq, G, dk, dv, window, n = 2, 1, 64, 64, 21, 90
+    kc, vc, bt = _paged(g, dt, [n], Hq, G, dk, dv)
+    far = 33
+    vc.mul_(0.2)
+    vc.view(-1, dv)[int(bt[0, far // 16]) * 16 + far % 16] = 100.0
+    qkv = _r(g, n, Hq * dk + G * (dk + dv), dt=dt)
+    a = (Hq, G, dk, dv, 0.01, window, True)
+    dev = [t.cuda() for t in (qkv, kc, vc, _i32([0, n]), _i32([0]), bt)]
+    got = H.window_attention_prefill(*dev, *a, mfma=True).cpu().float()
+    seen = got.abs().amax(1) > 2.0  # the spike weighs at least 100 / (window + 1); everything else stays below 1
+    assert seen.tolist() == [far <= r < far + window for r in range(n)]
+
+
+@pytest.mark.parametrize("dk,dv,Hq,G", [(64, 64, 4, 2), (128, 128, 8, 1), (24, 16, 2, 2), (32, 256, 4, 4), (128, 64, 4, 1)])
+@pytest.mark.parametrize("window", [7, 64, 100, 0])
+def test_window_decode_vec(dk, dv, Hq, G, window):
+    g = _g(10)
+    dt = torch.bfloat16
+    lens = [1, 64, 65, 200, 17]
+    kc, vc, bt = _paged(g, dt, lens, Hq, G, dk, dv)
+    q = _r(g, len(lens) + 1, Hq * dk + G * (dk + dv), dt=dt)
+    sl = _i32(lens + [0])
+    bt = torch.cat([bt, torch.zeros(1, bt.shape[1], dtype=torch.int32)])
+    a = (Hq, G, dk, dv, 1.0 / math.sqrt(dk), window, True)
+    want = H.window_attention_decode(q, kc, vc, bt, sl, *a)
+    dev = [t.cuda() for t in (q, kc, vc, bt, sl)]
+    torch.testing.assert_close(H.window_attention_decode(*dev, *a, vec=True).cpu().float(), want.float(), **_tol(dt))
+    torch.testing.assert_close(H.window_attention_decode(*dev, *a, vec=False).cpu().float(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("T,E,K,d,ff,il", [(45, 5, 2, 64, 96, False), (7, 8, 3, 128, 64, True), (300, 4, 2, 96, 128, True),
+                                           (700, 4, 2, 128, 128, True), (1, 3, 1, 32, 32, False)])
+def test_experts_matrix_core_paths(T, E, K, d, ff, il):
+    """16-row matrix-core kernel (gathered rows, ragged last tiles, interleaved gate / up) and, from
+    1024 sorted rows of an interleaved layer, the prefill tile GEMM."""
+    from k8s_llm_monitor_amd import ops
+
+    g = _g(11)
+    dt = torch.bfloat16
+    h = _r(g, T, d, dt=dt)
+    wr, bias = _r(g, E + 1, d, s=0.3), _r(g, E, s=0.3)
+    ids, w, gate = H.moe_router(h, wr, bias, E, K)
+    w13 = _r(g, E, 2 * ff, d, s=1 / math.sqrt(d), dt=dt)
+    w2 = _r(g, E, d, ff, s=1 / math.sqrt(ff), dt=dt)
+    sh = _r(g, T, d, dt=dt)
+    want = H.moe_experts(h, ids, w, w13, w2, sh, gate)
+    w13g = torch.stack([ops.interleave_gate_up(x) for x in w13]).contiguous() if il else w13
+    if il:  # the CPU form reads the interleaved layout too
+        torch.testing.assert_close(H.moe_experts(h, ids, w, w13g, w2, sh, gate, il=True), want, rtol=1e-5, atol=1e-5)
+    for mfma in (True, False):
+        got = H.moe_experts(h.cuda(), ids.cuda(), w.cuda(), w13g.cuda(), w2.cuda(), sh.cuda(), gate.cuda(), il=il, mfma=mfma)
+        torch.testing.assert_close(got.cpu(), want, **_tol(dt))
