@@ -72,7 +72,11 @@ __global__ __launch_bounds__(256) void conv_state_step_kernel(T* __restrict__ st
 
 // Workgroup = 4 waves = 64 values of p for one (segment, head); in a wave lanes are (p % 16,
 // chunk = lane / 16): chunk k holds states n in [k * NPT, (k + 1) * NPT) of its p in registers, and
-// the 4 partial sums of y meet through two xor-shuffles.
+// the 4 partial sums of y meet through two xor-shuffles.  The inputs of 16 tokens at a time (B, C
+// widened to fp32, x, and dt / the decay after softplus and exp) are staged in LDS by the whole
+// workgroup, so the token loop reads only LDS (16-byte reads; the chunks' rows are padded apart by
+// 4 floats so the 4 chunks of a wave hit different banks) and global latency is paid once per 16
+// tokens instead of once per token.
 template <typename T, int NPT>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, const T* __restrict__ xbc,
                                                        const T* __restrict__ proj, long p_stride, int dt_col,
@@ -81,47 +85,79 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, co
                                                        const float* __restrict__ d_skip, float* __restrict__ state,
                                                        const int* __restrict__ cu, const int* __restrict__ ctx,
                                                        const int* __restrict__ slot, int nh, int P, int N, int G) {
+  constexpr int TB = 16;
+  constexpr int CS = NPT + 4;
+  __shared__ __attribute__((aligned(16))) float Bs[TB][4 * CS];
+  __shared__ __attribute__((aligned(16))) float Cs[TB][4 * CS];
+  __shared__ float xs[TB][64];
+  __shared__ float dts[TB], dAs[TB];
   const int s = blockIdx.x, h = blockIdx.y;
   const int sl = slot[s];
   const int t0 = cu[s], t1 = cu[s + 1];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int p = blockIdx.z * 64 + wave * 16 + (lane & 15);
+  const int pl = wave * 16 + (lane & 15);
+  const int p = blockIdx.z * 64 + pl;
   if (sl < 0) {  // padding rows: defined output, no state
     if (p < P && lane < 16)
       for (int t = t0; t < t1; ++t) y[(long)t * nh * P + (long)h * P + p] = 0.f;
     return;
   }
   if (t1 <= t0) return;
-  const int n0 = (lane >> 4) * NPT;
+  const int chunk = lane >> 4, n0 = chunk * NPT;
   const bool live = p < P;
   const int g = h / (nh / G);
   const int inner = nh * P, C = inner + 2 * G * N;
+  for (int i = threadIdx.x; i < TB * 4 * CS; i += 256) {  // entries beyond N stay zero
+    (&Bs[0][0])[i] = 0.f;
+    (&Cs[0][0])[i] = 0.f;
+  }
   float S[NPT];
   float* sp = state + (((long)sl * nh + h) * N) * P + p;
   const bool carried = ctx[s] > 0;
 #pragma unroll
   for (int i = 0; i < NPT; ++i) S[i] = (carried && live && n0 + i < N) ? sp[(long)(n0 + i) * P] : 0.f;
   const float A = expf(a_log[h]), Dh = d_skip[h], bias = dt_bias[h];
-  for (int t = t0; t < t1; ++t) {
-    const T* row = xbc + (long)t * C;
-    const float raw = ldf(proj + (long)t * p_stride + dt_col + h) + bias;
-    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
-    const float dA = expf(-A * dt);
-    const float x = live ? ldf(row + (long)h * P + p) : 0.f;
-    const T* Bp = row + inner + (long)g * N + n0;
-    const T* Cp = Bp + (long)G * N;
-    const float dtx = dt * x;
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < NPT; ++i) {
-      if (n0 + i < N) {
-        S[i] = dA * S[i] + dtx * ldf(Bp + i);
-        acc += S[i] * ldf(Cp + i);
-      }
+  for (int tb = t0; tb < t1; tb += TB) {
+    const int nt = min(TB, t1 - tb);
+    __syncthreads();  // the previous tile is consumed (and the zero fill is done)
+    for (int i = threadIdx.x; i < nt * N; i += 256) {
+      const int tt = i / N, n = i - tt * N;
+      const T* row = xbc + (long)(tb + tt) * C + inner + (long)g * N + n;
+      const int off = (n / NPT) * CS + n % NPT;
+      Bs[tt][off] = ldf(row);
+      Cs[tt][off] = ldf(row + (long)G * N);
     }
-    acc += __shfl_xor(acc, 16, 64);
-    acc += __shfl_xor(acc, 32, 64);
-    if (live && lane < 16) y[(long)t * inner + (long)h * P + p] = acc + Dh * x;
+    for (int i = threadIdx.x; i < nt * 64; i += 256) {
+      const int tt = i >> 6, pp = i & 63;
+      const int pg = blockIdx.z * 64 + pp;
+      xs[tt][pp] = pg < P ? ldf(xbc + (long)(tb + tt) * C + (long)h * P + pg) : 0.f;
+    }
+    if (threadIdx.x < nt) {
+      const float raw = ldf(proj + (long)(tb + threadIdx.x) * p_stride + dt_col + h) + bias;
+      const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+      dts[threadIdx.x] = dt;
+      dAs[threadIdx.x] = expf(-A * dt);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float dA = dAs[tt], x = xs[tt][pl];
+      const float dtx = dts[tt] * x;
+      const float4* bp = reinterpret_cast<const float4*>(&Bs[tt][chunk * CS]);
+      const float4* cp = reinterpret_cast<const float4*>(&Cs[tt][chunk * CS]);
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < NPT / 4; ++i) {
+        const float4 bv = bp[i], cv = cp[i];
+        S[4 * i + 0] = dA * S[4 * i + 0] + dtx * bv.x;
+        S[4 * i + 1] = dA * S[4 * i + 1] + dtx * bv.y;
+        S[4 * i + 2] = dA * S[4 * i + 2] + dtx * bv.z;
+        S[4 * i + 3] = dA * S[4 * i + 3] + dtx * bv.w;
+        acc += S[4 * i + 0] * cv.x + S[4 * i + 1] * cv.y + S[4 * i + 2] * cv.z + S[4 * i + 3] * cv.w;
+      }
+      acc += __shfl_xor(acc, 16, 64);
+      acc += __shfl_xor(acc, 32, 64);
+      if (live && lane < 16) y[(long)(tb + tt) * inner + (long)h * P + p] = acc + Dh * x;
+    }
   }
   if (live) {
 #pragma unroll

@@ -152,13 +152,15 @@ __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y,
   }
 }
 
-// bf16 on the matrix cores (K a multiple of 32): one wave = 16 sorted rows x 64 output columns,
+// bf16 on the matrix cores (K a multiple of 32): one wave = 16 sorted rows x 16 NT output columns
+// (NT = 4; NT = 1 with a deeper unroll when there are few rows, so that a decode step's weight
+// stream is spread over four times as many waves),
 // v_mfma_f32_16x16x32_bf16 with both operands loaded straight from global memory as 16-byte
 // fragments (A = the gathered activation rows, B = weight rows, 8 consecutive k per lane).  Few
 // rows per expert (decode) make this a weight-streaming kernel: many small workgroups, no LDS.
 // ``il``: the gate / up rows are interleaved per 128 rows as [64 gate | 64 up] (the prefill tile
 // GEMM's pairing), else [all gate rows ; all up rows].
-template <bool SWIGLU>
+template <bool SWIGLU, int NT>
 __global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __restrict__ Y, const bf16_t* __restrict__ A,
                                                                   const bf16_t* __restrict__ W,
                                                                   const int* __restrict__ offsets,
@@ -175,35 +177,35 @@ __global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __rest
   if (e >= E) return;
   r0 += tile * 16;
   const int lane = threadIdx.x, c16 = lane & 15, quad = lane >> 4;
-  const int n0 = blockIdx.y * 64;
+  const int n0 = blockIdx.y * (16 * NT);
   const bf16_t* We = W + (long)e * w_es;
   const int arow = min(r0 + c16, r1 - 1);
   const long asrc = sorted_idx != nullptr ? sorted_idx[arow] / div : arow;
   const bf16_t* ap = A + asrc * Kd + 8 * quad;
-  const bf16_t* wg[4];
-  const bf16_t* wu[4];
+  const bf16_t* wg[NT];
+  const bf16_t* wu[NT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < NT; ++t) {
     const int n = min(n0 + 16 * t + c16, N - 1);
     const long g = SWIGLU && il ? (long)(n >> 6) * 128 + (n & 63) : n;
     wg[t] = We + g * Kd + 8 * quad;
     wu[t] = We + (SWIGLU ? (il ? g + 64 : (long)N + n) : 0) * Kd + 8 * quad;
   }
-  f32x4 acc[4], accu[4];
+  f32x4 acc[NT], accu[NT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) acc[t] = accu[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
+  for (int t = 0; t < NT; ++t) acc[t] = accu[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll(NT == 1 ? 8 : 2)
   for (int k0 = 0; k0 < Kd; k0 += 32) {
     const bf16x8 a = *reinterpret_cast<const bf16x8*>(ap + k0);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < NT; ++t) {
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, *reinterpret_cast<const bf16x8*>(wg[t] + k0), acc[t], 0, 0, 0);
       if (SWIGLU)
         accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, *reinterpret_cast<const bf16x8*>(wu[t] + k0), accu[t], 0, 0, 0);
     }
   }
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {  // acc[t][i]: row r0 + 4 quad + i, column n0 + 16 t + c16
+  for (int t = 0; t < NT; ++t) {  // acc[t][i]: row r0 + 4 quad + i, column n0 + 16 t + c16
     const int n = n0 + 16 * t + c16;
     if (n >= N) continue;
 #pragma unroll
@@ -257,13 +259,17 @@ int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* off
   if (rows <= 0) return 0;
   if (il && (!swiglu || N % 64)) return -1;
   if (!f32 && mfma && Kd % 32 == 0) {
-    const dim3 g16((unsigned)(rows / 16 + E), (unsigned)((N + 63) / 64));
-    if (swiglu)
-      hipLaunchKernelGGL(hy_grouped_gemm_mfma_kernel<true>, g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,
-                         (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il);
-    else
-      hipLaunchKernelGGL(hy_grouped_gemm_mfma_kernel<false>, g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,
-                         (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il);
+    const bool few = rows <= 512;  // a decode-sized step: one n-tile per wave
+    const dim3 g16((unsigned)(rows / 16 + E), (unsigned)(few ? (N + 15) / 16 : (N + 63) / 64));
+#define K8SLLM_GM(SW, NT)                                                                                        \
+  hipLaunchKernelGGL((hy_grouped_gemm_mfma_kernel<SW, NT>), g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,      \
+                     (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il)
+    if (swiglu) {
+      if (few) K8SLLM_GM(true, 1); else K8SLLM_GM(true, 4);
+    } else {
+      if (few) K8SLLM_GM(false, 1); else K8SLLM_GM(false, 4);
+    }
+#undef K8SLLM_GM
     return (int)hipGetLastError();
   }
   const dim3 grid((unsigned)(rows / TM + E), (unsigned)((N + TN - 1) / TN));

@@ -135,46 +135,51 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
                  n, h / (Hq / G), G, dk, dv, bs, scale, sink, q_s, p_s);
 }
 
-// bf16 decode with 16-byte loads: one wave per (sequence, kv head) serves all R = Hq / G query
-// heads of that kv head, so every cached key and value row is read once.  Scores: lane = key, the
-// lane walks its key row in 8-element pieces against the R queries held in LDS (fp32).  Values:
-// lane = (key subset, 8-dim piece); each lane accumulates its piece over its subset's keys and the
-// subsets meet through xor-shuffles once at the end.  Needs dk % 8 == 0 and dv / 8 a power of two.
+// bf16 decode with 16-byte loads: one workgroup (4 waves) per (sequence, kv head) serves all
+// R = Hq / G query heads of that kv head, so every cached key and value row is read once.  The
+// waves take the 64-key tiles of the window in turn (wave w: tiles w, w + 4, ...) and their partial
+// (maximum, denominator, output) triples are merged through LDS at the end; only wave 0 starts from
+// the sink's (0, 1).  Scores: lane = key, the lane walks its key row in 8-element pieces against the
+// R queries held in LDS (fp32).  Values: lane = (key subset, 8-dim piece); each lane accumulates its
+// piece over its subset's keys (the weights travel by lane shuffles) and the subsets meet through
+// xor-shuffles.  Needs dk % 8 == 0 and dv / 8 a power of two.
 template <int R>
-__global__ __launch_bounds__(64) void window_decode_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv,
-                                                               long q_stride, const bf16_t* __restrict__ k_cache,
-                                                               const bf16_t* __restrict__ v_cache,
-                                                               const int* __restrict__ block_tables, int bt_stride,
-                                                               const int* __restrict__ seq_lens, int Hq, int G, int dk,
-                                                               int dv, int bs, float scale, int window, int sink) {
+__global__ __launch_bounds__(256) void window_decode_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv,
+                                                                long q_stride, const bf16_t* __restrict__ k_cache,
+                                                                const bf16_t* __restrict__ v_cache,
+                                                                const int* __restrict__ block_tables, int bt_stride,
+                                                                const int* __restrict__ seq_lens, int Hq, int G, int dk,
+                                                                int dv, int bs, float scale, int window, int sink) {
   __shared__ __attribute__((aligned(16))) float q_s[R * kMaxDK];
-  __shared__ float p_s[R][64];
-  const int b = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  __shared__ float ml_s[4][R][2];
+  __shared__ float acc_s[4][R][64 * kMaxVC];
+  const int b = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = seq_lens[b];
-  const int DL = dv >> 3;            // lanes that cover the value dims, 8 each
+  const int DL = dv >> 3;  // lanes that cover the value dims, 8 each
   const int dg = lane & (DL - 1), ksub = lane / DL, KS = 64 / DL;
   bf16_t* o = out + (long)b * Hq * dv + (long)g * R * dv;
   if (n <= 0) {  // padding row of a decode bucket
-    for (int c = lane; c < R * dv; c += 64) o[c] = 0;
+    for (int c = threadIdx.x; c < R * dv; c += 256) o[c] = 0;
     return;
   }
   const bf16_t* q = qkv + (long)b * q_stride + (long)g * R * dk;
-  for (int c = lane; c < R * dk; c += 64) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * scale;
+  for (int c = threadIdx.x; c < R * dk; c += 256) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * scale;
   __syncthreads();
   const int* bt = block_tables + (long)b * bt_stride;
   const int lo = window > 0 ? max(0, n - window) : 0;
+  const bool first = sink && wave == 0;
   float m[R], l[R], acc[R][8];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    m[r] = sink ? 0.f : -INFINITY;
-    l[r] = sink ? 1.f : 0.f;
+    m[r] = first ? 0.f : -INFINITY;
+    l[r] = first ? 1.f : 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
   }
   const long krs = (long)G * dk, vrs = (long)G * dv;
-  for (int j0 = lo; j0 < n; j0 += 64) {
+  for (int j0 = lo + 64 * wave; j0 < n; j0 += 256) {
     const int j = j0 + lane;
-    float sc[R];
+    float sc[R], pw[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) sc[r] = 0.f;
     if (j < n) {
@@ -191,31 +196,30 @@ __global__ __launch_bounds__(64) void window_decode_vec_kernel(bf16_t* __restric
         }
       }
     }
-    __syncthreads();  // the previous tile's reads of p_s are done
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float s = j < n ? sc[r] : -INFINITY;
-      const float mt = fmaxf(m[r], wave_max(s));
-      const float p = j < n ? expf(s - mt) : 0.f;
+      const float sv = j < n ? sc[r] : -INFINITY;
+      const float mt = fmaxf(m[r], wave_max(sv));  // finite: the tile holds at least key j0
+      pw[r] = j < n ? expf(sv - mt) : 0.f;
       const float alpha = m[r] == -INFINITY ? 0.f : expf(m[r] - mt);
-      l[r] = l[r] * alpha + wave_sum(p);
+      l[r] = l[r] * alpha + wave_sum(pw[r]);
       m[r] = mt;
-      p_s[r][lane] = p;
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[r][i] *= alpha;
     }
-    __syncthreads();
     const int cnt = min(64, n - j0);
-    for (int i = ksub; i < cnt; i += KS) {
-      const int jj = j0 + i;
+    for (int i0 = 0; i0 < cnt; i0 += KS) {  // uniform trip count: the shuffles below need every lane
+      const int i = i0 + ksub;
+      const int jj = min(j0 + i, n - 1);
       float vv[8];
       unpack8(*reinterpret_cast<const uint4*>(v_cache + ((long)bt[jj / bs] * bs + jj % bs) * vrs + (long)g * dv + dg * 8),
               vv);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const float p = p_s[r][i];
+        const float pr = __shfl(pw[r], i & 63, 64);
+        const float pp = i < cnt ? pr : 0.f;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) acc[r][k] += p * vv[k];
+        for (int k = 0; k < 8; ++k) acc[r][k] += pp * vv[k];
       }
     }
   }
@@ -225,15 +229,27 @@ __global__ __launch_bounds__(64) void window_decode_vec_kernel(bf16_t* __restric
     for (int k = 0; k < 8; ++k) {
       float a = acc[r][k];
       for (int off = DL; off < 64; off <<= 1) a += __shfl_xor(a, off, 64);
-      acc[r][k] = a;
+      if (ksub == 0) acc_s[wave][r][dg * 8 + k] = a;
     }
-    if (ksub == 0) {
-      const float inv = l[r] > 0.f ? 1.f / l[r] : 0.f;
-      float w[8];
+    if (lane == 0) {
+      ml_s[wave][r][0] = m[r];
+      ml_s[wave][r][1] = l[r];
+    }
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < R * dv; c += 256) {
+    const int r = c / dv, dcol = c - r * dv;
+    float M = -INFINITY;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) w[k] = acc[r][k] * inv;
-      *reinterpret_cast<uint4*>(o + (long)r * dv + dg * 8) = pack8(w);
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_s[w][r][0]);
+    float L = 0.f, val = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = ml_s[w][r][0] == -INFINITY ? 0.f : expf(ml_s[w][r][0] - M);
+      L += ml_s[w][r][1] * f;
+      val += acc_s[w][r][dcol] * f;
     }
+    o[c] = f2bf(L > 0.f ? val / L : 0.f);
   }
 }
 
@@ -403,7 +419,7 @@ int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const voi
   if (!f32 && vec && dk % 8 == 0 && dv % 8 == 0 && DL >= 1 && DL <= 64 && (DL & (DL - 1)) == 0 && q_stride % 8 == 0 &&
       (R == 1 || R == 2 || R == 4 || R == 8)) {
 #define K8SLLM_WD(RR)                                                                                                  \
-  hipLaunchKernelGGL(window_decode_vec_kernel<RR>, dim3(B, G), dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,          \
+  hipLaunchKernelGGL(window_decode_vec_kernel<RR>, dim3(B, G), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)qkv,          \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_stride, seq_lens, Hq, G, \
                      dk, dv, bs, scale, window, sink)
     if (R == 1) K8SLLM_WD(1);
