@@ -28,7 +28,7 @@ int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int 
                         hipStream_t s);
 int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
                        const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
-                       const int* slot, int S, int nh, int P, int N, int G, int f32, hipStream_t s);
+                       const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode, hipStream_t s);
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
                      const float* bias, int E, int K, int rows_w, int f32, hipStream_t s);
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
@@ -175,7 +175,7 @@ void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int
 
 void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor cu, Tensor ctx,
                               Tensor block_tables, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
-                              int64_t window, bool sink, bool mfma) {
+                              int64_t window, bool sink, int64_t mfma) {
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
@@ -193,7 +193,7 @@ void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_c
   check(k8sllm_hy_window_prefill(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  cu.data_ptr<int>(), ctx.data_ptr<int>(), block_tables.data_ptr<int>(),
                                  (int)block_tables.stride(0), (int)S, T, (int)Hq, (int)G, (int)dk, (int)dv,
-                                 (int)k_cache.size(1), (float)scale, (int)window, sink, f, mfma, cur()),
+                                 (int)k_cache.size(1), (float)scale, (int)window, sink, f, (int)mfma, cur()),
         "window_attention_prefill");
 }
 
@@ -248,7 +248,8 @@ void conv_silu(Tensor out, Tensor proj, int64_t col0, Tensor cw, Tensor cb, Tens
 }
 
 void ssm_scan(Tensor y, Tensor xbc, Tensor proj, int64_t dt_col, Tensor dt_bias, Tensor a_log, Tensor d_skip,
-              Tensor state, Tensor cu, Tensor ctx, Tensor slot, int64_t nh, int64_t P, int64_t N, int64_t G) {
+              Tensor state, Tensor cu, Tensor ctx, Tensor slot, int64_t nh, int64_t P, int64_t N, int64_t G,
+              int64_t mode) {
   const int f = act(xbc, "xbc");
   same(proj, f, "proj");
   f32c(y, "y");
@@ -267,7 +268,7 @@ void ssm_scan(Tensor y, Tensor xbc, Tensor proj, int64_t dt_col, Tensor dt_bias,
   check(k8sllm_hy_ssm_scan(y.data_ptr<float>(), xbc.data_ptr(), proj.data_ptr(), proj.stride(0), (int)dt_col,
                            dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), d_skip.data_ptr<float>(),
                            state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(), slot.data_ptr<int>(),
-                           (int)ctx.numel(), (int)nh, (int)P, (int)N, (int)G, f, cur()),
+                           (int)ctx.numel(), T, (int)nh, (int)P, (int)N, (int)G, f, (int)mode, cur()),
         "ssm_scan");
 }
 

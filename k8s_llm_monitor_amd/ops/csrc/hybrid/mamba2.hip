@@ -166,6 +166,106 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, co
   }
 }
 
+// Long segments (prompts): the same recurrence with the state spread thinner - 8 states per lane,
+// CH = N / 8 lanes per value of p (reduced by xor-shuffles over neighbouring lanes), 64 / CH values
+// of p per wave.  Per token a lane then issues a quarter of the instructions of the mapping above
+// (at N = 128) and four times as many waves share the work, which is what bounds a prompt's scan:
+// the token loop is sequential per (sequence, head, p).  State rows are read and written with a
+// stride here, which is why single-token segments (decode) keep the mapping above.
+template <typename T, int CH>
+__global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ y, const T* __restrict__ xbc,
+                                                            const T* __restrict__ proj, long p_stride, int dt_col,
+                                                            const float* __restrict__ dt_bias,
+                                                            const float* __restrict__ a_log,
+                                                            const float* __restrict__ d_skip,
+                                                            float* __restrict__ state, const int* __restrict__ cu,
+                                                            const int* __restrict__ ctx, const int* __restrict__ slot,
+                                                            int nh, int P, int N, int G) {
+  constexpr int TB = 16, PW = 64 / CH, PB = 4 * PW;
+  constexpr int ROW = 8 * CH + (CH / 8) * 4 + 4;  // state n sits at n + 4 (n / 64): 64-float halves 4 banks apart
+  __shared__ __attribute__((aligned(16))) float Bs[TB][ROW];
+  __shared__ __attribute__((aligned(16))) float Cs[TB][ROW];
+  __shared__ float xs[TB][PB];
+  __shared__ float dts[TB], dAs[TB];
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int sl = slot[s];
+  const int t0 = cu[s], t1 = cu[s + 1];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int chunk = lane % CH, pl = wave * PW + lane / CH;
+  const int p = blockIdx.z * PB + pl;
+  const bool live = p < P;
+  const int inner = nh * P, C = inner + 2 * G * N;
+  if (sl < 0) {  // padding rows: defined output, no state
+    if (live && chunk == 0)
+      for (int t = t0; t < t1; ++t) y[(long)t * inner + (long)h * P + p] = 0.f;
+    return;
+  }
+  if (t1 <= t0) return;
+  const int n0 = chunk * 8;
+  const int g = h / (nh / G);
+  for (int i = threadIdx.x; i < TB * ROW; i += 256) {  // entries beyond N stay zero
+    (&Bs[0][0])[i] = 0.f;
+    (&Cs[0][0])[i] = 0.f;
+  }
+  float S[8];
+  float* sp = state + (((long)sl * nh + h) * N) * P + p;
+  const bool carried = ctx[s] > 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) S[i] = (carried && live && n0 + i < N) ? sp[(long)(n0 + i) * P] : 0.f;
+  const float A = expf(a_log[h]), Dh = d_skip[h], bias = dt_bias[h];
+  const int boff = n0 + (n0 >> 6) * 4;
+  for (int tb = t0; tb < t1; tb += TB) {
+    const int nt = min(TB, t1 - tb);
+    __syncthreads();  // the previous tile is consumed (and the zero fill is done)
+    for (int i = threadIdx.x; i < nt * N; i += 256) {
+      const int tt = i / N, n = i - tt * N;
+      const T* row = xbc + (long)(tb + tt) * C + inner + (long)g * N + n;
+      const int off = n + (n >> 6) * 4;
+      Bs[tt][off] = ldf(row);
+      Cs[tt][off] = ldf(row + (long)G * N);
+    }
+    for (int i = threadIdx.x; i < nt * PB; i += 256) {
+      const int tt = i / PB, pp = i % PB;
+      const int pg = blockIdx.z * PB + pp;
+      xs[tt][pp] = pg < P ? ldf(xbc + (long)(tb + tt) * C + (long)h * P + pg) : 0.f;
+    }
+    if (threadIdx.x < nt) {
+      const float raw = ldf(proj + (long)(tb + threadIdx.x) * p_stride + dt_col + h) + bias;
+      const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+      dts[threadIdx.x] = dt;
+      dAs[threadIdx.x] = expf(-A * dt);
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (int tt = 0; tt < nt; ++tt) {
+      const float dA = dAs[tt], x = xs[tt][pl];
+      const float dtx = dts[tt] * x;
+      const float4 b0 = *reinterpret_cast<const float4*>(&Bs[tt][boff]);
+      const float4 b1 = *reinterpret_cast<const float4*>(&Bs[tt][boff + 4]);
+      const float4 c0 = *reinterpret_cast<const float4*>(&Cs[tt][boff]);
+      const float4 c1 = *reinterpret_cast<const float4*>(&Cs[tt][boff + 4]);
+      S[0] = dA * S[0] + dtx * b0.x;
+      S[1] = dA * S[1] + dtx * b0.y;
+      S[2] = dA * S[2] + dtx * b0.z;
+      S[3] = dA * S[3] + dtx * b0.w;
+      S[4] = dA * S[4] + dtx * b1.x;
+      S[5] = dA * S[5] + dtx * b1.y;
+      S[6] = dA * S[6] + dtx * b1.z;
+      S[7] = dA * S[7] + dtx * b1.w;
+      float acc = S[0] * c0.x + S[1] * c0.y + S[2] * c0.z + S[3] * c0.w + S[4] * c1.x + S[5] * c1.y + S[6] * c1.z +
+                  S[7] * c1.w;
+#pragma unroll
+      for (int o = 1; o < CH; o <<= 1) acc += __shfl_xor(acc, o, 64);
+      if (live && chunk == 0) y[(long)(tb + tt) * inner + (long)h * P + p] = acc + Dh * x;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (n0 + i < N) sp[(long)(n0 + i) * P] = S[i];
+  }
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -173,7 +273,21 @@ using namespace k8sllm;
 template <typename T>
 static int launch_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
                        const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
-                       const int* slot, int S, int nh, int P, int N, int G, hipStream_t s) {
+                       const int* slot, int S, int nh, int P, int N, int G, int wide, hipStream_t s) {
+  if (wide && N > 8) {  // long segments: 8 states per lane
+#define K8SLLM_WIDE(CH)                                                                                              \
+  hipLaunchKernelGGL((ssm_scan_wide_kernel<T, CH>), dim3((unsigned)S, (unsigned)nh, (unsigned)((P + 256 / CH - 1) / (256 / CH))), \
+                     dim3(256), 0, s, y, (const T*)xbc, (const T*)proj, p_stride, dt_col, dt_bias, a_log, d_skip, state, \
+                     cu, ctx, slot, nh, P, N, G)
+    if (N <= 16) K8SLLM_WIDE(2);
+    else if (N <= 32) K8SLLM_WIDE(4);
+    else if (N <= 64) K8SLLM_WIDE(8);
+    else if (N <= 128) K8SLLM_WIDE(16);
+    else if (N <= 256) K8SLLM_WIDE(32);
+    else return -1;
+#undef K8SLLM_WIDE
+    return (int)hipGetLastError();
+  }
   const dim3 grid((unsigned)S, (unsigned)nh, (unsigned)((P + 63) / 64));
 #define K8SLLM_SCAN(NPT)                                                                                              \
   hipLaunchKernelGGL((ssm_scan_kernel<T, NPT>), grid, dim3(256), 0, s, y, (const T*)xbc, (const T*)proj, p_stride,    \
@@ -214,12 +328,14 @@ int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int 
 
 int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_stride, int dt_col, const float* dt_bias,
                        const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
-                       const int* slot, int S, int nh, int P, int N, int G, int f32, hipStream_t s) {
+                       const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode, hipStream_t s) {
   if (S <= 0) return 0;
   if (G < 1 || nh % G) return -1;
+  // mode 0: by the step's mean segment length (prompts: the thin mapping); 1 / 2: forced (tests)
+  const int wide = mode == 2 || (mode == 0 && T >= 32L * S);
   return f32 ? launch_scan<float>(y, xbc, proj, p_stride, dt_col, dt_bias, a_log, d_skip, state, cu, ctx, slot, S, nh,
-                                  P, N, G, s)
+                                  P, N, G, wide, s)
              : launch_scan<bf16_t>(y, xbc, proj, p_stride, dt_col, dt_bias, a_log, d_skip, state, cu, ctx, slot, S,
-                                   nh, P, N, G, s);
+                                   nh, P, N, G, wide, s);
 }
 }

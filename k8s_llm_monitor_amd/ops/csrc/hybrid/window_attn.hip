@@ -261,101 +261,157 @@ __global__ __launch_bounds__(256) void window_decode_vec_kernel(bf16_t* __restri
 //                             the lane, 4 keys per lane: the C layout of S^T IS the B layout of P^T),
 //                             A = V^T read back transposed from an LDS copy of the 16-key V tile
 // With the query on the lane the running maximum, denominator and the rescale of O are lane-local
-// (two xor-shuffles per reduction).  Scores, weights and sums are fp32; P is rounded to bf16 for
-// the PV product.
-template <int DK, int DV>
+// (two xor-shuffles per reduction).  Scores, weights and sums are fp32 (base-2 exponentials: the
+// scale carries log2 e); P is rounded to bf16 for the PV product.
+template <int DK, int DV, int QT>
 __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv, long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
-    const int* __restrict__ block_tables, int bt_stride, int S, int Hq, int G, int bs, float scale, int window,
+    const int* __restrict__ block_tables, int bt_stride, int S, int Hq, int G, int bsh, float scale, int window,
     int sink) {
+  // pages hold 1 << bsh tokens; scores live in the base-2 domain (scale * log2 e folded in) so that
+  // every exponential is one v_exp_f32
+  const int bsm = (1 << bsh) - 1;
+  const float sc2 = scale * 1.44269504088896341f;
   constexpr int VP = DV + 16;  // LDS row pitch: the 4 key rows of a fragment read land 8 banks apart
+  constexpr int QB = 16 * QT;  // query rows per wave: QT tiles of 16 share every K and V^T fragment
   __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * VP];
   int tile = blockIdx.x, s = 0, n = 0;
-  for (; s < S; ++s) {  // q-tiles are numbered segment by segment
+  for (; s < S; ++s) {  // q-blocks are numbered segment by segment
     n = cu[s + 1] - cu[s];
-    const int nt = (n + 15) >> 4;
+    const int nt = (n + QB - 1) / QB;
     if (tile < nt) break;
     tile -= nt;
   }
   if (s >= S) return;
-  const int q0 = tile * 16, nq = min(16, n - q0);
+  const int q0 = tile * QB, nq = min(QB, n - q0);
   const int h = blockIdx.y, g = h / (Hq / G);
   const int lane = threadIdx.x, c16 = lane & 15, quad = lane >> 4;
   const int* bt = block_tables + (long)s * bt_stride;
   const int row0 = cu[s] + q0, p0 = ctx[s] + q0;
-  const int myq = min(c16, nq - 1);
-  const int my_p = p0 + myq;
-  const int my_lo = window > 0 ? max(0, my_p - window + 1) : 0;
-  const bool q_live = c16 < nq;
-  bf16x8 qf[DK / 32];
-  const bf16_t* qrow = qkv + (long)(row0 + myq) * q_stride + (long)h * DK;
+  int my_p[QT], my_lo[QT];
+  bool q_live[QT];
+  bf16x8 qf[QT][DK / 32];
+  f32x4 oacc[QT][DV / 16];
+  float m[QT], l[QT];
 #pragma unroll
-  for (int ks = 0; ks < DK / 32; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * quad);
-  f32x4 oacc[DV / 16];
+  for (int t = 0; t < QT; ++t) {
+    const int myq = min(16 * t + c16, nq - 1);
+    my_p[t] = p0 + myq;
+    my_lo[t] = window > 0 ? max(0, my_p[t] - window + 1) : 0;
+    q_live[t] = 16 * t + c16 < nq;
+    const bf16_t* qrow = qkv + (long)(row0 + myq) * q_stride + (long)h * DK;
 #pragma unroll
-  for (int dt = 0; dt < DV / 16; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+    for (int ks = 0; ks < DK / 32; ++ks) qf[t][ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * quad);
+#pragma unroll
+    for (int dt = 0; dt < DV / 16; ++dt) oacc[t][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m[t] = sink ? 0.f : -INFINITY;
+    l[t] = sink ? 1.f : 0.f;
+  }
   const int lo_t = window > 0 ? max(0, p0 - window + 1) : 0, hi = p0 + nq;
   const long krs = (long)G * DK, vrs = (long)G * DV;
-  for (int j0 = lo_t & ~15; j0 < hi; j0 += 16) {
-    const int jk = min(j0 + c16, hi - 1);
-    const bf16_t* krow = k_cache + ((long)bt[jk / bs] * bs + jk % bs) * krs + (long)g * DK;
-    f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+  // Register double buffer: while tile j0 is computed, the K fragments and V pieces of tile j0 + 16
+  // are in flight, and the page ids of tile j0 + 32 behind them (no load waits on a load issued in
+  // the same iteration).  A lane's V pieces: piece c = lane + 64 u of the 16 x DV tile.
+  constexpr int NV = DV / 32, CPK = DV / 8;  // pieces per lane, 16-byte pieces per key
+  const bf16_t* kbase = k_cache + (long)g * DK + 8 * quad;
+  const bf16_t* vbase = v_cache + (long)g * DV + (lane % CPK) * 8;
+  int vkey[NV];
 #pragma unroll
-    for (int ks = 0; ks < DK / 32; ++ks)
-      sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + 32 * ks + 8 * quad),
-                                                     qf[ks], sacc, 0, 0, 0);
-    float sv[4], tmax = -INFINITY;
+  for (int u = 0; u < NV; ++u) vkey[u] = (lane + 64 * u) / CPK;
+  const int jfirst = lo_t & ~15;
+  auto kpage = [&](int j0) { return bt[min(j0 + c16, hi - 1) >> bsh]; };
+  auto vpage = [&](int j0, int u) { return bt[min(j0 + vkey[u], hi - 1) >> bsh]; };
+  int pk_n = kpage(jfirst), pv_n[NV];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, query c16
-      const int j = j0 + 4 * quad + i;
-      sv[i] = (q_live && j >= my_lo && j <= my_p) ? sacc[i] * scale : -INFINITY;
-      tmax = fmaxf(tmax, sv[i]);
+  for (int u = 0; u < NV; ++u) pv_n[u] = vpage(jfirst, u);
+  bf16x8 kf_n[DK / 32];
+  uint4 vf_n[NV];
+  auto issue = [&](int j0) {  // loads of tile j0 from the page ids in pk_n / pv_n
+    const bf16_t* krow = kbase + (((long)pk_n << bsh) + (min(j0 + c16, hi - 1) & bsm)) * krs;
+#pragma unroll
+    for (int ks = 0; ks < DK / 32; ++ks) kf_n[ks] = *reinterpret_cast<const bf16x8*>(krow + 32 * ks);
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+      vf_n[u] = *reinterpret_cast<const uint4*>(vbase + (((long)pv_n[u] << bsh) + (min(j0 + vkey[u], hi - 1) & bsm)) * vrs);
+  };
+  issue(jfirst);
+  pk_n = kpage(jfirst + 16);
+#pragma unroll
+  for (int u = 0; u < NV; ++u) pv_n[u] = vpage(jfirst + 16, u);
+  for (int j0 = jfirst; j0 < hi; j0 += 16) {
+    bf16x8 kf[DK / 32];
+#pragma unroll
+    for (int ks = 0; ks < DK / 32; ++ks) kf[ks] = kf_n[ks];
+    // LDS traffic of a one-wave workgroup needs no s_barrier: a wave's LDS instructions execute in
+    // issue order, so the compiler-level barrier (no reordering across it) is all that is needed
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < NV; ++u) *reinterpret_cast<uint4*>(&Vs[vkey[u] * VP + (lane % CPK) * 8]) = vf_n[u];
+    __builtin_amdgcn_wave_barrier();
+    if (j0 + 16 < hi) {
+      issue(j0 + 16);
+      pk_n = kpage(j0 + 32);
+#pragma unroll
+      for (int u = 0; u < NV; ++u) pv_n[u] = vpage(j0 + 32, u);
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float mn = fmaxf(m, tmax);
-    const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
-    float pv[4], ps = 0.f;
+    s16x4 pb[QT];
+    float alpha[QT];
+    bool rescale[QT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      pv[i] = sv[i] == -INFINITY ? 0.f : expf(sv[i] - mn);
-      ps += pv[i];
-    }
-    ps += __shfl_xor(ps, 16, 64);
-    ps += __shfl_xor(ps, 32, 64);
-    l = l * alpha + ps;
-    m = mn;
-    s16x4 pb;
+    for (int t = 0; t < QT; ++t) {
+      f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pb[i] = (short)f2bf(pv[i]);
-    __syncthreads();  // one wave per workgroup: the previous tile's fragment reads are done
-    for (int c = lane; c < 16 * (DV / 8); c += 64) {
-      const int key = c / (DV / 8), dc = c % (DV / 8);
-      const int jv = min(j0 + key, hi - 1);
-      const bf16_t* vrow = v_cache + ((long)bt[jv / bs] * bs + jv % bs) * vrs + (long)g * DV;
-      *reinterpret_cast<uint4*>(&Vs[key * VP + dc * 8]) = *reinterpret_cast<const uint4*>(vrow + dc * 8);
+      for (int ks = 0; ks < DK / 32; ++ks) sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[t][ks], sacc, 0, 0, 0);
+      float sv[4], tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, query 16 t + c16
+        const int j = j0 + 4 * quad + i;
+        sv[i] = (q_live[t] && j >= my_lo[t] && j <= my_p[t]) ? sacc[i] * sc2 : -INFINITY;
+        tmax = fmaxf(tmax, sv[i]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float mn = fmaxf(m[t], tmax);
+      alpha[t] = m[t] == -INFINITY ? 0.f : exp2f(m[t] - mn);
+      float ps = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = sv[i] == -INFINITY ? 0.f : exp2f(sv[i] - mn);
+        ps += pv;
+        pb[t][i] = (short)f2bf(pv);
+      }
+      ps += __shfl_xor(ps, 16, 64);
+      ps += __shfl_xor(ps, 32, 64);
+      l[t] = l[t] * alpha[t] + ps;
+      m[t] = mn;
+      rescale[t] = __any(alpha[t] != 1.f);
     }
-    __syncthreads();
 #pragma unroll
     for (int dt = 0; dt < DV / 16; ++dt) {
       s16x4 a;
 #pragma unroll
       for (int i = 0; i < 4; ++i) a[i] = (short)Vs[(4 * quad + i) * VP + 16 * dt + c16];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
-      oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dt], 0, 0, 0);
+      for (int t = 0; t < QT; ++t) {
+        if (rescale[t]) {  // wave-uniform: once the running maxima settle, most tiles skip this
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
+        }
+        oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[t], oacc[t][dt], 0, 0, 0);
+      }
     }
   }
-  if (q_live) {  // oacc[dt][i] = O[q = c16][d = 16 dt + 4 quad + i]
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    bf16_t* orow = out + (long)(row0 + c16) * Hq * DV + (long)h * DV;
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    if (!q_live[t]) continue;  // oacc[t][dt][i] = O[q = 16 t + c16][d = 16 dt + 4 quad + i]
+    const float inv = l[t] > 0.f ? 1.f / l[t] : 0.f;
+    bf16_t* orow = out + (long)(row0 + 16 * t + c16) * Hq * DV + (long)h * DV;
 #pragma unroll
     for (int dt = 0; dt < DV / 16; ++dt) {
       uint2 w;
-      w.x = pack2(oacc[dt][0] * inv, oacc[dt][1] * inv);
-      w.y = pack2(oacc[dt][2] * inv, oacc[dt][3] * inv);
+      w.x = pack2(oacc[t][dt][0] * inv, oacc[t][dt][1] * inv);
+      w.y = pack2(oacc[t][dt][2] * inv, oacc[t][dt][3] * inv);
       *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * quad) = w;
     }
   }
@@ -386,16 +442,28 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
   if (T <= 0 || S <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
   // bf16 with matrix-core head sizes and 16-byte aligned rows: the MFMA kernel
-  if (!f32 && mfma && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
-    const dim3 grid((unsigned)(T / 16 + S), (unsigned)Hq);
-#define K8SLLM_WP(DK, DV)                                                                                             \
-  hipLaunchKernelGGL((window_prefill_mfma_kernel<DK, DV>), grid, dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,      \
+  int bsh = 0;
+  while ((1 << bsh) < bs) ++bsh;
+  if (!f32 && mfma && (1 << bsh) == bs && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
+    // query rows per wave: 16, or 32 once the step is large enough to fill the chip that way (64
+    // shares each K / V fragment among more rows but leaves one wave per SIMD: slower); mfma = 16 /
+    // 32 / 64 forces one (tests, measurements)
+    const int qrows = mfma >= 16 ? mfma : (T * Hq >= 64 * 1024 ? 32 : 16);
+    const dim3 grid((unsigned)(T / qrows + S), (unsigned)Hq);
+#define K8SLLM_WP(DK, DV, QT)                                                                                          \
+  hipLaunchKernelGGL((window_prefill_mfma_kernel<DK, DV, QT>), grid, dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,  \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, block_tables, bt_stride, S, Hq, \
-                     G, bs, scale, window, sink)
-    if (dk == 64 && dv == 64) K8SLLM_WP(64, 64);
-    else if (dk == 64) K8SLLM_WP(64, 128);
-    else if (dv == 64) K8SLLM_WP(128, 64);
-    else K8SLLM_WP(128, 128);
+                     G, bsh, scale, window, sink)
+#define K8SLLM_WPQ(DK, DV)                                       \
+  if (qrows == 64) K8SLLM_WP(DK, DV, 4);                         \
+  else if (qrows == 32) K8SLLM_WP(DK, DV, 2);                    \
+  else K8SLLM_WP(DK, DV, 1)
+    if (mfma >= 16 && mfma != 16 && mfma != 32 && mfma != 64) return -1;
+    if (dk == 64 && dv == 64) { K8SLLM_WPQ(64, 64); }
+    else if (dk == 64) { K8SLLM_WPQ(64, 128); }
+    else if (dv == 64) { K8SLLM_WPQ(128, 64); }
+    else { K8SLLM_WPQ(128, 128); }
+#undef K8SLLM_WPQ
 #undef K8SLLM_WP
     return (int)hipGetLastError();
   }

@@ -130,12 +130,13 @@ def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, sin
 
 def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu: torch.Tensor,
                              ctx: torch.Tensor, block_tables: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int,
-                             scale: float, window: int, sink: bool, mfma: bool = True) -> torch.Tensor:
+                             scale: float, window: int, sink: bool, mfma: int = 1) -> torch.Tensor:
     """Attention of the step's prompt chunks over the paged cache (which already holds their own
     keys): row r of segment s at position p = ctx[s] + r sees positions max(0, p - window + 1) .. p
     (``window`` 0: all of 0 .. p).  ``sink``: the softmax denominator has one more term exp(0) that
     carries no value.  Scores and weights are fp32.  Returns [T, Hq*dv].  GPU, bf16, head sizes
-    64 / 128: the matrix-core kernel (``mfma=False``: the any-size wave-per-row kernel)."""
+    64 / 128: the matrix-core kernel, 16 query rows per wave or 32 in large steps (``mfma`` 0: the
+    any-size wave-per-row kernel; 16 / 32 / 64: that many rows per wave whatever the step's size)."""
     T = qkv.shape[0]
     if not qkv.is_cuda:
         out = torch.empty(T, Hq * dv, dtype=qkv.dtype)
@@ -154,7 +155,7 @@ def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: 
         return out
     out = torch.empty(T, Hq * dv, dtype=qkv.dtype, device=qkv.device)
     native().window_attention_prefill(out, qkv, k_cache, v_cache, cu, ctx, block_tables, Hq, Hkv, dk, dv, float(scale),
-                                      int(window), bool(sink), bool(mfma))
+                                      int(window), bool(sink), int(mfma))
     return out
 
 
@@ -220,7 +221,7 @@ def conv_silu(proj: torch.Tensor, col0: int, C: int, conv_w: torch.Tensor, conv_
 
 def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
              d_skip: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor,
-             seg_slot: torch.Tensor, nh: int, P: int, N: int, G: int) -> torch.Tensor:
+             seg_slot: torch.Tensor, nh: int, P: int, N: int, G: int, mode: int = 0) -> torch.Tensor:
     """The selective state-space recurrence, fp32, token by token within each segment:
 
         dt = softplus(proj[t, dt_col + h] + dt_bias[h]);  S <- exp(-exp(a_log[h]) dt) S + dt B_t x_t^T
@@ -228,7 +229,8 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.
 
     ``xbc`` [T, nh*P | G*N | G*N] holds x, B, C (head h reads group h // (nh / G)); ``state``
     [slots, nh, N, P] fp32 is read at the segment's start (zero where seg_ctx is 0) and written
-    back at its end.  Returns y [T, nh*P] fp32."""
+    back at its end.  Returns y [T, nh*P] fp32.  GPU: two lane mappings of the same arithmetic,
+    chosen by the step's mean segment length (``mode`` 1 / 2 forces the decode / the prompt one)."""
     T = xbc.shape[0]
     if not xbc.is_cuda:
         y = torch.zeros(T, nh * P, dtype=torch.float32)
@@ -252,7 +254,8 @@ def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.
             state[slot] = S
         return y
     y = torch.empty(T, nh * P, dtype=torch.float32, device=xbc.device)
-    native().ssm_scan(y, xbc, proj, int(dt_col), dt_bias, a_log, d_skip, state, seg_cu, seg_ctx, seg_slot, nh, P, N, G)
+    native().ssm_scan(y, xbc, proj, int(dt_col), dt_bias, a_log, d_skip, state, seg_cu, seg_ctx, seg_slot, nh, P, N, G,
+                      int(mode))
     return y
 
 

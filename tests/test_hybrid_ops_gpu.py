@@ -134,7 +134,7 @@ def test_conv_silu_with_state(dt, taps):
 @pytest.mark.parametrize("nh,P,N,G", [(4, 24, 12, 2), (2, 80, 40, 1), (3, 16, 130, 3)])
 def test_ssm_scan_with_state(dt, nh, P, N, G):
     g = _g(6)
-    new, ctx, slot = [6, 1, 3], [0, 9, 2], [1, 3, 0]
+    new, ctx, slot = [6, 1, 3, 40, 2], [0, 9, 2, 0, 1], [1, 3, 0, 2, -1]
     T = sum(new)
     inner = nh * P
     xbc = _r(g, T, inner + 2 * G * N, s=0.7, dt=dt)
@@ -144,10 +144,12 @@ def test_ssm_scan_with_state(dt, nh, P, N, G):
     cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
     s_c, s_g = state.clone(), state.clone().cuda()
     want = H.ssm_scan(xbc, proj, 11, dtb, alog, dsk, s_c, cu, _i32(ctx), _i32(slot), nh, P, N, G)
-    got = H.ssm_scan(xbc.cuda(), proj.cuda(), 11, dtb.cuda(), alog.cuda(), dsk.cuda(), s_g, cu.cuda(), _i32(ctx).cuda(),
-                     _i32(slot).cuda(), nh, P, N, G)
-    torch.testing.assert_close(got.cpu(), want, rtol=2e-5, atol=2e-5)
-    torch.testing.assert_close(s_g.cpu(), s_c, rtol=2e-5, atol=2e-5)
+    for mode in (1, 2):  # both lane mappings
+        s_g = state.clone().cuda()
+        got = H.ssm_scan(xbc.cuda(), proj.cuda(), 11, dtb.cuda(), alog.cuda(), dsk.cuda(), s_g, cu.cuda(),
+                         _i32(ctx).cuda(), _i32(slot).cuda(), nh, P, N, G, mode=mode)
+        torch.testing.assert_close(got.cpu(), want, rtol=2e-5, atol=2e-5)
+        torch.testing.assert_close(s_g.cpu(), s_c, rtol=2e-5, atol=2e-5)
 
 
 @pytest.mark.parametrize("dt", DT)
@@ -179,7 +181,7 @@ def test_window_prefill_mfma(dk, dv, Hq, G, window, sink):
     windows at, below and above the tile size."""
     g = _g(8)
     dt = torch.bfloat16
-    ctx, new = [0, 40, 130, 7, 16], [37, 5, 33, 1, 16]
+    ctx, new = [0, 40, 130, 7, 16, 3], [37, 5, 33, 1, 16, 150]
     lens = [c + n for c, n in zip(ctx, new)]
     kc, vc, bt = _paged(g, dt, lens, Hq, G, dk, dv)
     cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
@@ -187,10 +189,9 @@ def test_window_prefill_mfma(dk, dv, Hq, G, window, sink):
     a = (Hq, G, dk, dv, 1.0 / math.sqrt(dk), window, sink)
     want = H.window_attention_prefill(qkv, kc, vc, cu, _i32(ctx), bt, *a)
     dev = [t.cuda() for t in (qkv, kc, vc, cu, _i32(ctx), bt)]
-    got = H.window_attention_prefill(*dev, *a, mfma=True)
-    plain = H.window_attention_prefill(*dev, *a, mfma=False)
-    torch.testing.assert_close(plain.cpu().float(), want.float(), **_tol(dt))
-    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+    for mode in (0, 1, 16, 32, 64):  # wave-per-row kernel, automatic, 16 / 32 / 64 query rows per wave
+        got = H.window_attention_prefill(*dev, *a, mfma=mode)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
 
 
 def test_window_prefill_mfma_sees_exactly_the_window():
@@ -205,9 +206,10 @@ def test_window_prefill_mfma_sees_exactly_the_window():
     qkv = _r(g, n, Hq * dk + G * (dk + dv), dt=dt)
     a = (Hq, G, dk, dv, 0.01, window, True)
     dev = [t.cuda() for t in (qkv, kc, vc, _i32([0, n]), _i32([0]), bt)]
-    got = H.window_attention_prefill(*dev, *a, mfma=True).cpu().float()
-    seen = got.abs().amax(1) > 2.0  # the spike weighs at least 100 / (window + 1); everything else stays below 1
-    assert seen.tolist() == [far <= r < far + window for r in range(n)]
+    for mode in (16, 32, 64):
+        got = H.window_attention_prefill(*dev, *a, mfma=mode).cpu().float()
+        seen = got.abs().amax(1) > 2.0  # the spike weighs at least 100 / (window + 1); everything else stays below 1
+        assert seen.tolist() == [far <= r < far + window for r in range(n)]
 
 
 @pytest.mark.parametrize("dk,dv,Hq,G", [(64, 64, 4, 2), (128, 128, 8, 1), (24, 16, 2, 2), (32, 256, 4, 4), (128, 64, 4, 1)])
