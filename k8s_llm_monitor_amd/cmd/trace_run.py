@@ -53,7 +53,7 @@ def main(argv=None) -> int:
     dev = a.device or ("cuda" if torch.cuda.is_available() else "cpu")
     nb = (a.max_tokens + BLOCK_SIZE - 1) // BLOCK_SIZE
     eng = LLMEngine(EngineConfig(model=a.model, weights=a.model, dtype=a.dtype, max_num_seqs=MAX_SEQS,
-                                 max_model_len=1 << 30, num_blocks=nb, use_graphs=a.graphs, keep_logits=True,
+                                 max_model_len=1 << 30, num_blocks=nb, use_graphs=a.graphs, keep_logits=True, sample=False,
                                  prefix_caching=False, pipeline=False), device=dev)
     if getattr(eng.model, "uses_tile_gemm", False) and dev != "cpu":
         from ..ops import build

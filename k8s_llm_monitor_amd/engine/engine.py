@@ -69,6 +69,7 @@ class EngineConfig:
     # weights instead of the seeded random init (models/checkpoint.py); None = random init
     weights: Optional[str] = None
     keep_logits: bool = False  # keep each step's logits on the device (trace replay; RunnerConfig.keep_logits)
+    sample: bool = True  # False: decode steps stop at the logits (trace replay; RunnerConfig.sample)
 
 
 class _View:
@@ -105,7 +106,8 @@ class LLMEngine:
                                  pstate=self.ps, weights=cfg.weights)
         self.runner = ModelRunner(self.model, RunnerConfig(
             max_num_seqs=cfg.max_num_seqs, max_model_len=cfg.max_model_len, kv_cache_gb=cfg.kv_cache_gb,
-            num_blocks=cfg.num_blocks, use_graphs=cfg.use_graphs, seed=cfg.seed, keep_logits=cfg.keep_logits))
+            num_blocks=cfg.num_blocks, use_graphs=cfg.use_graphs, seed=cfg.seed, keep_logits=cfg.keep_logits,
+            sample=cfg.sample))
         self.blocks = BlockManager(self.runner.num_blocks, prefix_caching=cfg.prefix_caching,
                                    state_slots=self.runner.num_state_slots)
         self.sched = Scheduler(SchedulerConfig(max_num_seqs=cfg.max_num_seqs,

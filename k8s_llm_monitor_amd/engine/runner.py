@@ -39,6 +39,9 @@ class RunnerConfig:
     # keep every step's logits on the device (ModelRunner.last_logits / DecodeHandle.logits): the
     # trace replayer reads them; serving leaves it off
     keep_logits: bool = False
+    # False: decode steps stop at the logits (nothing is sampled, d_out keeps its contents) - for
+    # callers that feed every token themselves (trace replay)
+    sample: bool = True
 
 
 class ModelRunner:
@@ -332,7 +335,8 @@ class ModelRunner:
                 self.d_logits = torch.zeros(self.B, logits.shape[1], dtype=torch.float32, device=self.device)
             self.d_logits[:b].copy_(logits)
             self.last_logits = self.d_logits[:b]
-        self._sample(logits, self.d_temp[:b], self.d_topk[:b], self.d_topp[:b], out=self.d_out[:b])
+        if self.cfg.sample:
+            self._sample(logits, self.d_temp[:b], self.d_topk[:b], self.d_topp[:b], out=self.d_out[:b])
 
     def capture_graphs(self, buckets: Optional[list[int]] = None) -> None:
         if not (self.is_gpu and self.cfg.use_graphs):

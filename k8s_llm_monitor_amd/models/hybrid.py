@@ -77,6 +77,7 @@ class WindowAttention:
         self.window = int(m.get("mask.size", 0) or 0)
         self.sink = bool(m.get("sink", True))
         self.eps = eps
+        self.fast = 1  # 0: the any-size attention kernels only (ops.hybrid mfma / vec switches; tests)
         nq, nk, nv = self.H * self.dk, self.G * self.dk, self.G * self.dv
         s = 1.0 / math.sqrt(d)
         self.wqkv = torch.cat([p.get(prefix + "q", (nq, d), s), p.get(prefix + "k", (nk, d), s),
@@ -100,13 +101,14 @@ class WindowAttention:
         hops.qk_norm_cache(qkv, self.qn, self.kn, self.eps, H, G, dk, dv, kc, vc, meta.slot_mapping)
         args = (H, G, dk, dv, self.scale, self.window, self.sink)
         if not meta.is_prefill:
-            o = hops.window_attention_decode(qkv, kc, vc, meta.block_tables, meta.seq_lens, *args)
+            o = hops.window_attention_decode(qkv, kc, vc, meta.block_tables, meta.seq_lens, *args, vec=bool(self.fast))
         else:
             nd = meta.num_decode
             o = hops.window_attention_prefill(qkv[nd:], kc, vc, meta.cu_seqlens, meta.ctx_start, meta.block_tables,
-                                              *args)
+                                              *args, mfma=self.fast)
             if nd:  # a mixed step: the single decode tokens in front go through the decode kernel
-                od = hops.window_attention_decode(qkv[:nd], kc, vc, meta.dec_block_tables, meta.dec_seq_lens, *args)
+                od = hops.window_attention_decode(qkv[:nd], kc, vc, meta.dec_block_tables, meta.dec_seq_lens, *args,
+                                                  vec=bool(self.fast))
                 o = torch.cat([od, o])
         return F.linear(o, self.wo)
 

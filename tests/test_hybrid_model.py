@@ -414,6 +414,35 @@ def test_gpu_bf16_no_experts_is_within_rounding():
 
 
 @pytest.mark.gpu
+def test_gpu_matrix_core_paths_in_model():
+    """Head sizes and expert shapes that take the matrix-core kernels (MFMA prefill attention,
+    vector decode attention, MFMA / tile grouped expert GEMMs, the prompt mapping of the scan): every
+    cut of a prompt agrees with the oracle, and no worse than the any-size kernels do."""
+    cfg = make_cfg([with_mlp(attn(4, 2, 64, 64, 20, 0.125), moe(4, 2, 128, 128)), ssm(4, 32, 16, 2, 4, 2),
+                    with_mlp(attn(2, 1, 128, 128, 33, 0.09), None)], width=128, vocab=97, loop=(0, 2, 2))
+    t = toks(600, cfg["vocab"], 4)  # 1200 routed rows in the whole-prompt step: the tile GEMM
+    w = O.random_weights(cfg, 6)
+    want = O.forward(cfg, w, t)
+    scale = float(want.pow(2).mean().sqrt())
+
+    def rms(got):
+        return float((got.double() - want).pow(2).mean().sqrt()) / scale
+
+    errs = {}
+    for fast in (1, 0):
+        rig = Rig(cfg, w=w, device="cuda", dtype=torch.bfloat16, num_blocks=80)
+        assert rig.model.uses_tile_gemm
+        for m in rig.model.mixers:
+            m.fast = fast
+        for name, cuts in (("whole", [600]), ("cut", [100, 37, 2, 300, 64]), ("decode", [560])):
+            got = rig.run_cut("a", t, cuts)
+            close_most(got, want, 0.06)
+            errs[(fast, name)] = rms(got)
+    for name in ("whole", "cut", "decode"):
+        assert errs[(1, name)] <= 1.5 * errs[(0, name)] + 0.005, errs
+
+
+@pytest.mark.gpu
 def test_gpu_greedy_generation_with_graphs():
     eng = LLMEngine(EngineConfig(model="dunesun-tiny", max_num_seqs=4, max_model_len=256, num_blocks=64,
                                  dtype="float32", max_prefill_tokens=32, mixed_prefill_tokens=16), device="cuda")
