@@ -419,7 +419,8 @@ def test_gpu_matrix_core_paths_in_model():
     vector decode attention, MFMA / tile grouped expert GEMMs, the prompt mapping of the scan): every
     cut of a prompt agrees with the oracle, and no worse than the any-size kernels do."""
     cfg = make_cfg([with_mlp(attn(4, 2, 64, 64, 20, 0.125), moe(4, 2, 128, 128)), ssm(4, 32, 16, 2, 4, 2),
-                    with_mlp(attn(2, 1, 128, 128, 33, 0.09), None)], width=128, vocab=97, loop=(0, 2, 2))
+                    with_mlp(attn(2, 1, 128, 128, 33, 0.09), None)], width=128, vocab=97, loop=(0, 2, 2),
+                   max_positions=640)
     t = toks(600, cfg["vocab"], 4)  # 1200 routed rows in the whole-prompt step: the tile GEMM
     w = O.random_weights(cfg, 6)
     want = O.forward(cfg, w, t)
