@@ -24,6 +24,23 @@ __device__ __forceinline__ float ld_any(const void* p, int dt, long i) {
   return dt == 2 ? reinterpret_cast<const float*>(p)[i] : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
 }
 
+// 8 consecutive elements (16-byte aligned for bf16, 32-byte for fp32) as floats, and back
+__device__ __forceinline__ void load8(const bf16_t* p, float* f) { unpack8(*reinterpret_cast<const uint4*>(p), f); }
+__device__ __forceinline__ void load8(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+  f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* f) { *reinterpret_cast<uint4*>(p) = pack8(f); }
+__device__ __forceinline__ void store8(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
+}
+__device__ __forceinline__ void load8_any(const void* p, int dt, long i, float* f) {
+  if (dt == 2) load8(reinterpret_cast<const float*>(p) + i, f);
+  else load8(reinterpret_cast<const bf16_t*>(p) + i, f);
+}
+
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
 
 // the segment that holds row r: largest s with cu[s] <= r (cu has S + 1 entries, cu[0] = 0)

@@ -44,6 +44,46 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(T* __restrict__ out, con
   stf(out + (long)row * C + c, silu_f(acc));
 }
 
+// The same with 8 channels per thread (16 / 32-byte accesses): channel count, column offset and
+// row strides multiples of 8.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_silu_vec8_kernel(T* __restrict__ out, const T* __restrict__ proj,
+                                                             long stride, int col0, int C, const float* __restrict__ cw,
+                                                             const float* __restrict__ cb, int taps,
+                                                             const T* __restrict__ state, const int* __restrict__ cu,
+                                                             const int* __restrict__ ctx, const int* __restrict__ slot,
+                                                             int S) {
+  const int row = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  const int s = find_segment(cu, S, row);
+  const int sl = slot[s];
+  float acc[8], x[8];
+  if (sl < 0) {  // padding row: defined output, no state
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    store8(out + (long)row * C + c, acc);
+    return;
+  }
+  const int r = row - cu[s];
+  const bool carried = ctx[s] > 0;
+  load8(cb + c, acc);
+  for (int j = 0; j < taps; ++j) {
+    const int i = r - (taps - 1) + j;
+    if (i >= 0)
+      load8(proj + (long)(row - (taps - 1) + j) * stride + col0 + c, x);
+    else if (carried)
+      load8(state + ((long)sl * (taps - 1) + (taps - 1 + i)) * C + c, x);
+    else
+      continue;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] += cw[(long)(c + k) * taps + j] * x[k];
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) acc[k] = silu_f(acc[k]);
+  store8(out + (long)row * C + c, acc);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_step_kernel(T* __restrict__ state, const T* __restrict__ proj,
                                                               long stride, int col0, int C, int taps,
@@ -120,13 +160,15 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(float* __restrict__ y, co
   for (int tb = t0; tb < t1; tb += TB) {
     const int nt = min(TB, t1 - tb);
     __syncthreads();  // the previous tile is consumed (and the zero fill is done)
-    for (int i = threadIdx.x; i < nt * N; i += 256) {
+#pragma unroll 8
+    for (int i = threadIdx.x; i < nt * N; i += 256) {  // unrolled: the independent loads go out together
       const int tt = i / N, n = i - tt * N;
       const T* row = xbc + (long)(tb + tt) * C + inner + (long)g * N + n;
       const int off = (n / NPT) * CS + n % NPT;
       Bs[tt][off] = ldf(row);
       Cs[tt][off] = ldf(row + (long)G * N);
     }
+#pragma unroll 4
     for (int i = threadIdx.x; i < nt * 64; i += 256) {
       const int tt = i >> 6, pp = i & 63;
       const int pg = blockIdx.z * 64 + pp;
@@ -217,7 +259,8 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ 
   for (int tb = t0; tb < t1; tb += TB) {
     const int nt = min(TB, t1 - tb);
     __syncthreads();  // the previous tile is consumed (and the zero fill is done)
-    for (int i = threadIdx.x; i < nt * N; i += 256) {
+#pragma unroll 8
+    for (int i = threadIdx.x; i < nt * N; i += 256) {  // unrolled: the independent loads go out together
       const int tt = i / N, n = i - tt * N;
       const T* row = xbc + (long)(tb + tt) * C + inner + (long)g * N + n;
       const int off = n + (n >> 6) * 4;
@@ -310,15 +353,25 @@ int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int 
   if (T <= 0 || S <= 0) return 0;
   if (taps < 1 || taps > kMaxTaps) return -1;
   const dim3 g1((unsigned)T, (unsigned)((C + 255) / 256)), g2((unsigned)S, (unsigned)((C + 255) / 256));
+  const bool v8 = C % 8 == 0 && col0 % 8 == 0 && stride % 8 == 0;
+  const dim3 g8((unsigned)T, (unsigned)((C / 8 + 255) / 256));
   if (f32) {
-    hipLaunchKernelGGL(conv_silu_kernel<float>, g1, dim3(256), 0, s, (float*)out, (const float*)proj, stride, col0, C,
-                       cw, cb, taps, (const float*)state, cu, ctx, slot, S);
+    if (v8)
+      hipLaunchKernelGGL(conv_silu_vec8_kernel<float>, g8, dim3(256), 0, s, (float*)out, (const float*)proj, stride, col0,
+                         C, cw, cb, taps, (const float*)state, cu, ctx, slot, S);
+    else
+      hipLaunchKernelGGL(conv_silu_kernel<float>, g1, dim3(256), 0, s, (float*)out, (const float*)proj, stride, col0, C,
+                         cw, cb, taps, (const float*)state, cu, ctx, slot, S);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_step_kernel<float>, g2, dim3(256), 0, s, (float*)state, (const float*)proj, stride,
                          col0, C, taps, cu, ctx, slot);
   } else {
-    hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, g1, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)proj, stride, col0,
-                       C, cw, cb, taps, (const bf16_t*)state, cu, ctx, slot, S);
+    if (v8)
+      hipLaunchKernelGGL(conv_silu_vec8_kernel<bf16_t>, g8, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)proj, stride,
+                         col0, C, cw, cb, taps, (const bf16_t*)state, cu, ctx, slot, S);
+    else
+      hipLaunchKernelGGL(conv_silu_kernel<bf16_t>, g1, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)proj, stride, col0,
+                         C, cw, cb, taps, (const bf16_t*)state, cu, ctx, slot, S);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_step_kernel<bf16_t>, g2, dim3(256), 0, s, (bf16_t*)state, (const bf16_t*)proj,
                          stride, col0, C, taps, cu, ctx, slot);

@@ -13,21 +13,64 @@ namespace k8sllm {
 constexpr int kMaxE = 256;
 constexpr int kMaxK = 16;
 
-template <typename T>
+// NACC > 0: at most NACC weight rows - every thread reads its columns of h once and keeps all the
+// rows' partial dot products in registers (h is the large operand; the fp32 weight rows stay in L1);
+// NACC == 0: any number of rows, one wave per row in turn.
+template <typename T, int NACC>
 __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                         float* __restrict__ gate, const T* __restrict__ h, int d,
                                                         const float* __restrict__ wr, const float* __restrict__ bias,
                                                         int E, int K, int rows_w) {
   __shared__ float lg[kMaxE + 1];
+  __shared__ float part[4][NACC > 0 ? NACC : 1];
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* x = h + t * d;
-  for (int e = wave; e < rows_w; e += 4) {
-    const float* w = wr + (long)e * d;
-    float a = 0.f;
-    for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
-    a = wave_sum(a);
-    if (lane == 0) lg[e] = e < E ? a + bias[e] : a;
+  if (NACC > 0) {
+    float acc[NACC > 0 ? NACC : 1];
+#pragma unroll
+    for (int e = 0; e < NACC; ++e) acc[e] = 0.f;
+    if ((d & 7) == 0) {  // 8 columns per thread and trip: 16-byte loads of h, 32 bytes of each weight row
+      for (int c = threadIdx.x * 8; c < d; c += 2048) {
+        float xv[8];
+        load8(x + c, xv);
+#pragma unroll
+        for (int e = 0; e < NACC; ++e)
+          if (e < rows_w) {
+            const float4 wa = *reinterpret_cast<const float4*>(wr + (long)e * d + c);
+            const float4 wb = *reinterpret_cast<const float4*>(wr + (long)e * d + c + 4);
+            acc[e] += xv[0] * wa.x + xv[1] * wa.y + xv[2] * wa.z + xv[3] * wa.w + xv[4] * wb.x + xv[5] * wb.y +
+                      xv[6] * wb.z + xv[7] * wb.w;
+          }
+      }
+    } else {
+#pragma unroll 4
+      for (int c = threadIdx.x; c < d; c += 256) {
+        const float xv = ldf(x + c);
+#pragma unroll
+        for (int e = 0; e < NACC; ++e)
+          if (e < rows_w) acc[e] += xv * wr[(long)e * d + c];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < NACC; ++e) {
+      const float v = wave_sum(acc[e]);
+      if (lane == 0) part[wave][e] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < rows_w) {
+      const int e = threadIdx.x;
+      const float a = part[0][e] + part[1][e] + part[2][e] + part[3][e];
+      lg[e] = e < E ? a + bias[e] : a;
+    }
+  } else {
+    for (int e = wave; e < rows_w; e += 4) {
+      const float* w = wr + (long)e * d;
+      float a = 0.f;
+      for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
+      a = wave_sum(a);
+      if (lane == 0) lg[e] = e < E ? a + bias[e] : a;
+    }
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -243,12 +286,15 @@ int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, i
                      const float* bias, int E, int K, int rows_w, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (E > kMaxE || K > kMaxK || K > E || K < 1 || rows_w < E || rows_w > E + 1) return -1;
-  if (f32)
-    hipLaunchKernelGGL(hy_router_kernel<float>, dim3(T), dim3(256), 0, s, ids, wts, gate, (const float*)h, d, wr, bias,
-                       E, K, rows_w);
-  else
-    hipLaunchKernelGGL(hy_router_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids, wts, gate, (const bf16_t*)h, d, wr,
-                       bias, E, K, rows_w);
+#define K8SLLM_RT(T_, NACC)                                                                                       \
+  hipLaunchKernelGGL((hy_router_kernel<T_, NACC>), dim3(T), dim3(256), 0, s, ids, wts, gate, (const T_*)h, d, wr, bias, \
+                     E, K, rows_w)
+  if (f32) {
+    if (rows_w <= 9) K8SLLM_RT(float, 9); else if (rows_w <= 17) K8SLLM_RT(float, 17); else K8SLLM_RT(float, 0);
+  } else {
+    if (rows_w <= 9) K8SLLM_RT(bf16_t, 9); else if (rows_w <= 17) K8SLLM_RT(bf16_t, 17); else K8SLLM_RT(bf16_t, 0);
+  }
+#undef K8SLLM_RT
   return (int)hipGetLastError();
 }
 

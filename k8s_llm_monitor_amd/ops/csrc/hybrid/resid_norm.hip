@@ -31,6 +31,46 @@ __global__ __launch_bounds__(256) void add_norm_kernel(T* __restrict__ out, floa
   const long row = blockIdx.x;
   float* r = residual + row * d;
   float ss = 0.f;
+  if ((d & 7) == 0) {  // 8 columns per thread and trip, 16 / 32-byte accesses
+    for (int c = threadIdx.x * 8; c < d; c += 2048) {
+      float x[8], a[8];
+      load8(r + c, x);
+      if (t0) {
+        load8_any(a0, t0, row * d + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += a[i];
+      }
+      if (t1) {
+        load8_any(a1, t1, row * d + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += a[i];
+      }
+      if (t2) {
+        load8_any(a2, t2, row * d + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += a[i];
+      }
+      if (vec != nullptr) {
+        load8(vec + c, a);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += a[i];
+      }
+      store8(r + c, x);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+    }
+    ss = block_sum<256>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int c = threadIdx.x * 8; c < d; c += 2048) {  // each thread re-reads what it wrote
+      float x[8], g[8];
+      load8(r + c, x);
+      load8(w + c, g);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] *= inv * (one_plus ? 1.f + g[i] : g[i]);
+      store8(out + row * d + c, x);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < d; c += 256) {
     float x = r[c];
     if (t0) x += ld_any(a0, t0, row * d + c);

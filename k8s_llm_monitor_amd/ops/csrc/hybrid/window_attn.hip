@@ -135,35 +135,36 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
                  n, h / (Hq / G), G, dk, dv, bs, scale, sink, q_s, p_s);
 }
 
-// bf16 decode with 16-byte loads: one workgroup (4 waves) per (sequence, kv head) serves all
+// bf16 decode with 16-byte loads: one workgroup (NW = 8 waves; 4 for 8 query heads per kv head,
+// whose merge buffers would not fit otherwise) per (sequence, kv head) serves all
 // R = Hq / G query heads of that kv head, so every cached key and value row is read once.  The
-// waves take the 64-key tiles of the window in turn (wave w: tiles w, w + 4, ...) and their partial
+// waves take the 64-key tiles of the window in turn (wave w: tiles w, w + NW, ...) and their partial
 // (maximum, denominator, output) triples are merged through LDS at the end; only wave 0 starts from
 // the sink's (0, 1).  Scores: lane = key, the lane walks its key row in 8-element pieces against the
 // R queries held in LDS (fp32).  Values: lane = (key subset, 8-dim piece); each lane accumulates its
 // piece over its subset's keys (the weights travel by lane shuffles) and the subsets meet through
 // xor-shuffles.  Needs dk % 8 == 0 and dv / 8 a power of two.
-template <int R>
-__global__ __launch_bounds__(256) void window_decode_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv,
+template <int R, int NW>
+__global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv,
                                                                 long q_stride, const bf16_t* __restrict__ k_cache,
                                                                 const bf16_t* __restrict__ v_cache,
                                                                 const int* __restrict__ block_tables, int bt_stride,
                                                                 const int* __restrict__ seq_lens, int Hq, int G, int dk,
                                                                 int dv, int bs, float scale, int window, int sink) {
   __shared__ __attribute__((aligned(16))) float q_s[R * kMaxDK];
-  __shared__ float ml_s[4][R][2];
-  __shared__ float acc_s[4][R][64 * kMaxVC];
+  __shared__ float ml_s[NW][R][2];
+  __shared__ float acc_s[NW][R][64 * kMaxVC];
   const int b = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = seq_lens[b];
   const int DL = dv >> 3;  // lanes that cover the value dims, 8 each
   const int dg = lane & (DL - 1), ksub = lane / DL, KS = 64 / DL;
   bf16_t* o = out + (long)b * Hq * dv + (long)g * R * dv;
   if (n <= 0) {  // padding row of a decode bucket
-    for (int c = threadIdx.x; c < R * dv; c += 256) o[c] = 0;
+    for (int c = threadIdx.x; c < R * dv; c += 64 * NW) o[c] = 0;
     return;
   }
   const bf16_t* q = qkv + (long)b * q_stride + (long)g * R * dk;
-  for (int c = threadIdx.x; c < R * dk; c += 256) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * scale;
+  for (int c = threadIdx.x; c < R * dk; c += 64 * NW) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * scale;
   __syncthreads();
   const int* bt = block_tables + (long)b * bt_stride;
   const int lo = window > 0 ? max(0, n - window) : 0;
@@ -177,22 +178,32 @@ __global__ __launch_bounds__(256) void window_decode_vec_kernel(bf16_t* __restri
     for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
   }
   const long krs = (long)G * dk, vrs = (long)G * dv;
-  for (int j0 = lo + 64 * wave; j0 < n; j0 += 256) {
+  for (int j0 = lo + 64 * wave; j0 < n; j0 += 64 * NW) {
     const int j = j0 + lane;
     float sc[R], pw[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) sc[r] = 0.f;
     if (j < n) {
       const bf16_t* kp = k_cache + ((long)bt[j / bs] * bs + j % bs) * krs + (long)g * dk;
-      for (int c = 0; c < dk; c += 8) {
-        float kv[8];
-        unpack8(*reinterpret_cast<const uint4*>(kp + c), kv);
+      for (int c0 = 0; c0 < dk; c0 += 64) {  // 8 pieces of the key row in flight at a time
+        uint4 kq[8];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const float4 qa = *reinterpret_cast<const float4*>(&q_s[r * kMaxDK + c]);
-          const float4 qb = *reinterpret_cast<const float4*>(&q_s[r * kMaxDK + c + 4]);
-          sc[r] += kv[0] * qa.x + kv[1] * qa.y + kv[2] * qa.z + kv[3] * qa.w + kv[4] * qb.x + kv[5] * qb.y +
-                   kv[6] * qb.z + kv[7] * qb.w;
+        for (int u = 0; u < 8; ++u)
+          if (c0 + 8 * u < dk) kq[u] = *reinterpret_cast<const uint4*>(kp + c0 + 8 * u);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int c = c0 + 8 * u;
+          if (c < dk) {
+            float kv[8];
+            unpack8(kq[u], kv);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const float4 qa = *reinterpret_cast<const float4*>(&q_s[r * kMaxDK + c]);
+              const float4 qb = *reinterpret_cast<const float4*>(&q_s[r * kMaxDK + c + 4]);
+              sc[r] += kv[0] * qa.x + kv[1] * qa.y + kv[2] * qa.z + kv[3] * qa.w + kv[4] * qb.x + kv[5] * qb.y +
+                       kv[6] * qb.z + kv[7] * qb.w;
+            }
+          }
         }
       }
     }
@@ -208,18 +219,25 @@ __global__ __launch_bounds__(256) void window_decode_vec_kernel(bf16_t* __restri
       for (int i = 0; i < 8; ++i) acc[r][i] *= alpha;
     }
     const int cnt = min(64, n - j0);
-    for (int i0 = 0; i0 < cnt; i0 += KS) {  // uniform trip count: the shuffles below need every lane
-      const int i = i0 + ksub;
-      const int jj = min(j0 + i, n - 1);
-      float vv[8];
-      unpack8(*reinterpret_cast<const uint4*>(v_cache + ((long)bt[jj / bs] * bs + jj % bs) * vrs + (long)g * dv + dg * 8),
-              vv);
+    for (int i0 = 0; i0 < cnt; i0 += 4 * KS) {  // uniform trip counts: the shuffles below need every lane
+      uint4 vq[4];  // 4 value pieces in flight at a time
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const float pr = __shfl(pw[r], i & 63, 64);
-        const float pp = i < cnt ? pr : 0.f;
+      for (int u = 0; u < 4; ++u) {
+        const int jj = min(j0 + i0 + u * KS + ksub, n - 1);
+        vq[u] = *reinterpret_cast<const uint4*>(v_cache + ((long)bt[jj / bs] * bs + jj % bs) * vrs + (long)g * dv + dg * 8);
+      }
 #pragma unroll
-        for (int k = 0; k < 8; ++k) acc[r][k] += pp * vv[k];
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * KS + ksub;
+        float vv[8];
+        unpack8(vq[u], vv);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const float pr = __shfl(pw[r], i & 63, 64);
+          const float pp = i < cnt ? pr : 0.f;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc[r][k] += pp * vv[k];
+        }
       }
     }
   }
@@ -237,14 +255,14 @@ __global__ __launch_bounds__(256) void window_decode_vec_kernel(bf16_t* __restri
     }
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < R * dv; c += 256) {
+  for (int c = threadIdx.x; c < R * dv; c += 64 * NW) {
     const int r = c / dv, dcol = c - r * dv;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_s[w][r][0]);
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, ml_s[w][r][0]);
     float L = 0.f, val = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float f = ml_s[w][r][0] == -INFINITY ? 0.f : expf(ml_s[w][r][0] - M);
       L += ml_s[w][r][1] * f;
       val += acc_s[w][r][dcol] * f;
@@ -487,7 +505,8 @@ int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const voi
   if (!f32 && vec && dk % 8 == 0 && dv % 8 == 0 && DL >= 1 && DL <= 64 && (DL & (DL - 1)) == 0 && q_stride % 8 == 0 &&
       (R == 1 || R == 2 || R == 4 || R == 8)) {
 #define K8SLLM_WD(RR)                                                                                                  \
-  hipLaunchKernelGGL(window_decode_vec_kernel<RR>, dim3(B, G), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)qkv,          \
+  hipLaunchKernelGGL((window_decode_vec_kernel<RR, (RR == 8 ? 4 : 8)>), dim3(B, G), dim3(RR == 8 ? 256 : 512), 0, s,     \
+                     (bf16_t*)out, (const bf16_t*)qkv,                                                                  \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_stride, seq_lens, Hq, G, \
                      dk, dv, bs, scale, window, sink)
     if (R == 1) K8SLLM_WD(1);

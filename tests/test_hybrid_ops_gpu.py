@@ -28,9 +28,10 @@ def _i32(x):
 
 
 @pytest.mark.parametrize("dt", DT)
-def test_embed_pos_and_add_norm(dt):
+@pytest.mark.parametrize("d", [72, 70, 2304])  # 8-wide vector path, scalar path, several trips per thread
+def test_embed_pos_and_add_norm(dt, d):
     g = _g(1)
-    V, d, T = 50, 72, 7
+    V, T = 50, 7
     emb, pos = _r(g, V, d, dt=dt), _r(g, 40, d, dt=dt)
     ids, p = torch.randint(0, V, (T,), generator=g, dtype=torch.int32), torch.randint(0, 40, (T,), generator=g, dtype=torch.int32)
     src, prev = _i32([-1, 2, -1, 0, -1, -1, 1]), _i32([5, 6, 7])
@@ -112,12 +113,12 @@ def test_qk_norm_cache(dt):
 
 @pytest.mark.parametrize("dt", DT)
 @pytest.mark.parametrize("taps", [1, 2, 4])
-def test_conv_silu_with_state(dt, taps):
+@pytest.mark.parametrize("C,col0,pad", [(70, 9, 5), (72, 8, 8)])  # scalar path / 8 channels per thread
+def test_conv_silu_with_state(dt, taps, C, col0, pad):
     g = _g(5)
-    C, col0 = 70, 9
     new, ctx, slot = [5, 1, 2, 3], [0, 4, 7, 0], [2, 0, -1, 3]
     T = sum(new)
-    proj = _r(g, T, col0 + C + 5, dt=dt)
+    proj = _r(g, T, col0 + C + pad, dt=dt)
     cw, cb = _r(g, C, taps, s=0.5), _r(g, C, s=0.1)
     state = _r(g, 4, max(1, taps - 1), C, dt=dt)
     cu = _i32([0] + torch.tensor(new).cumsum(0).tolist())
@@ -153,7 +154,7 @@ def test_ssm_scan_with_state(dt, nh, P, N, G):
 
 
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("E,K,shared", [(5, 2, True), (24, 4, False), (70, 1, True)])
+@pytest.mark.parametrize("E,K,shared", [(5, 2, True), (12, 3, True), (24, 4, False), (70, 1, True)])
 def test_router_and_experts(dt, E, K, shared):
     g = _g(7)
     T, d, ff = 45, 72, 40
