@@ -10,7 +10,8 @@ branch sums of layer i are folded into layer i+1's norm launch (ops.hybrid.add_n
 fused add + RMSNorm of the Llama path.  Looped layers: pass t starts with ``x += loop.step[t]``
 (and ``x += embedding output`` for t > 0), folded into the same launch.
 
-State: an attention run owns paged K / V (``[blocks, 16, heads*dim]``, activation dtype); a
+State: an attention run owns paged K ``[blocks, 16, heads*dim]`` and V ``[blocks, heads, vdim, 16]``
+(activation dtype); a
 Mamba-2 run owns per-sequence slots - the fp32 state ``[slots, heads, N, P]`` and the last
 taps-1 convolution inputs.  Every RUN (a looped layer counts once per pass) has its own.
 
@@ -88,7 +89,7 @@ class WindowAttention:
 
     def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
         return {"k": torch.zeros(num_blocks, BLOCK, self.G * self.dk, dtype=dtype, device=device),
-                "v": torch.zeros(num_blocks, BLOCK, self.G * self.dv, dtype=dtype, device=device)}
+                "v": torch.zeros(num_blocks, self.G, self.dv, BLOCK, dtype=dtype, device=device)}
 
     def cache_bytes(self, esize: int) -> tuple:
         """(bytes per page, bytes per state slot)."""

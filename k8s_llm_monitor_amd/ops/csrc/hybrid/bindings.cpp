@@ -15,7 +15,7 @@ int k8sllm_hy_gated_group_norm(void* out, const float* y, const void* z, long z_
                                int n, int groups, float eps, int f32, hipStream_t s);
 int k8sllm_hy_swiglu(void* out, const void* gu, long rows, int f, int f32, hipStream_t s);
 int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float* kw, float eps, long T, int nq,
-                            int nk, int nv, void* k_cache, void* v_cache, const int* slots, int f32, hipStream_t s);
+                            int nk, int nv, void* k_cache, void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
 int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                              const int* cu, const int* ctx, const int* block_tables, int bt_stride, int S, long T,
                              int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink, int f32,
@@ -142,10 +142,17 @@ void swiglu(Tensor out, Tensor gu) {
   check(k8sllm_hy_swiglu(out.data_ptr(), gu.data_ptr(), gu.size(0), (int)(gu.size(1) / 2), f, cur()), "swiglu");
 }
 
-// pages [blocks, bs, width]
+// key pages [blocks, bs, width]
 void pages(const Tensor& c, int f, int64_t width, const char* n) {
   same(c, f, n);
   TORCH_CHECK(c.dim() == 3 && c.is_contiguous() && c.size(2) == width, n, " must be [blocks, block, heads*dim]");
+}
+// value pages [blocks, G, dv, bs] matching the key pages' block count and size
+void vpages(const Tensor& c, const Tensor& k, int f, int64_t G, int64_t dv) {
+  same(c, f, "v_cache");
+  TORCH_CHECK(c.dim() == 4 && c.is_contiguous() && c.size(0) == k.size(0) && c.size(1) == G && c.size(2) == dv &&
+                  c.size(3) == k.size(1),
+              "v_cache must be [blocks, kv_heads, vdim, block]");
 }
 
 void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int64_t G, int64_t dk, int64_t dv,
@@ -161,15 +168,15 @@ void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int
   if (k_cache.has_value()) {
     TORCH_CHECK(v_cache.has_value() && slots.has_value(), "k_cache, v_cache and slot_mapping come together");
     pages(*k_cache, f, nk, "k_cache");
-    pages(*v_cache, f, nv, "v_cache");
-    TORCH_CHECK(k_cache->size(0) == v_cache->size(0) && k_cache->size(1) == v_cache->size(1), "k / v pages differ");
+    vpages(*v_cache, *k_cache, f, G, dv);
     sp = iptr(slots, "slot_mapping");
     TORCH_CHECK(slots->numel() >= qkv.size(0), "slot_mapping [T]");
     kc = k_cache->data_ptr();
     vc = v_cache->data_ptr();
   }
   check(k8sllm_hy_qk_norm_cache(qkv.data_ptr(), qkv.stride(0), qw.data_ptr<float>(), kw.data_ptr<float>(), (float)eps,
-                                qkv.size(0), (int)nq, (int)nk, (int)nv, kc, vc, sp, f, cur()),
+                                qkv.size(0), (int)nq, (int)nk, (int)nv, kc, vc, sp,
+                                k_cache.has_value() ? (int)k_cache->size(1) : 16, f, cur()),
         "qk_norm_cache");
 }
 
@@ -179,7 +186,7 @@ void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_c
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
-  pages(v_cache, f, G * dv, "v_cache");
+  vpages(v_cache, k_cache, f, G, dv);
   i32c(cu, "cu");
   i32c(ctx, "ctx");
   TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == torch::kInt32 && block_tables.dim() == 2 &&
@@ -203,7 +210,7 @@ void window_attention_decode(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_ca
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
-  pages(v_cache, f, G * dv, "v_cache");
+  vpages(v_cache, k_cache, f, G, dv);
   i32c(seq_lens, "seq_lens");
   TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == torch::kInt32 && block_tables.dim() == 2 &&
                   block_tables.stride(1) == 1,

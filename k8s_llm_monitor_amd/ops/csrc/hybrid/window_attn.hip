@@ -2,7 +2,8 @@
 //   qk_norm_cache             whole-projection RMSNorm of q and of k in place, k / v -> pages
 //   window_attention_prefill  one wave per (chunk row, query head)
 //   window_attention_decode   one wave per (sequence, query head)
-// Pages: k_cache [blocks][BS][G*dk], v_cache [blocks][BS][G*dv]; a sequence's page list is a row of
+// Pages: k_cache [blocks][BS][G*dk] (a token's keys contiguous), v_cache [blocks][G][dv][BS] (a value
+// dim's BS tokens contiguous: the layout the PV products read along); a sequence's page list is a row of
 // block_tables.  Row at position p sees positions max(0, p - window + 1) .. p (window 0: 0 .. p).
 // The sink is one more softmax term with score 0 and no value: the running maximum starts at 0 and
 // the running denominator at 1.  Scores, weights and the output accumulation are fp32.
@@ -18,7 +19,7 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(T* __restrict__ qkv,
                                                             const float* __restrict__ qw,
                                                             const float* __restrict__ kw, float eps, int nq, int nk,
                                                             int nv, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                                            const int* __restrict__ slots) {
+                                                            const int* __restrict__ slots, int bs) {
   __shared__ float red[4];
   const long t = blockIdx.x;
   T* row = qkv + t * stride;
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(T* __restrict__ qkv,
     if (slot >= 0) k_cache[slot * nk + c] = row[nq + c];
   }
   if (slot >= 0)
-    for (int c = threadIdx.x; c < nv; c += 256) v_cache[slot * nv + c] = row[nq + nk + c];
+    for (int c = threadIdx.x; c < nv; c += 256) v_cache[((slot / bs) * nv + c) * bs + slot % bs] = row[nq + nk + c];
 }
 
 // One wave: query q (dk values at q_row) against cached positions [lo, hi) of one kv head.
@@ -83,7 +84,7 @@ __device__ __forceinline__ void attend_wave(T* __restrict__ out_row, const T* __
       if (dcol < dv)
         for (int i = 0; i < n; ++i) {
           const int jj = j0 + i;
-          a += p_s[i] * ldf(v_cache + ((long)bt[jj / bs] * bs + jj % bs) * vrow + (long)g * dv + dcol);
+          a += p_s[i] * ldf(v_cache + ((long)bt[jj / bs] * vrow + (long)g * dv + dcol) * bs + jj % bs);
         }
       acc[c] = a;
     }
@@ -135,29 +136,28 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
                  n, h / (Hq / G), G, dk, dv, bs, scale, sink, q_s, p_s);
 }
 
-// bf16 decode with 16-byte loads: one workgroup (NW = 8 waves; 4 for 8 query heads per kv head,
-// whose merge buffers would not fit otherwise) per (sequence, kv head) serves all
-// R = Hq / G query heads of that kv head, so every cached key and value row is read once.  The
-// waves take the 64-key tiles of the window in turn (wave w: tiles w, w + NW, ...) and their partial
-// (maximum, denominator, output) triples are merged through LDS at the end; only wave 0 starts from
-// the sink's (0, 1).  Scores: lane = key, the lane walks its key row in 8-element pieces against the
-// R queries held in LDS (fp32).  Values: lane = (key subset, 8-dim piece); each lane accumulates its
-// piece over its subset's keys (the weights travel by lane shuffles) and the subsets meet through
-// xor-shuffles.  Needs dk % 8 == 0 and dv / 8 a power of two.
+// bf16 decode with 16-byte loads, 16-token pages: one workgroup (NW = 8 waves; 4 for 8 query heads
+// per kv head, whose merge buffers would not fit otherwise) per (sequence, kv head) serves all
+// R = Hq / G query heads of that kv head, so every cached key and value is read once.  The waves take
+// the window's 64-key tiles (aligned to 64, i.e. four whole pages) in turn and their partial (maximum,
+// denominator, output) triples are merged through LDS at the end; only wave 0 starts from the sink's
+// (0, 1).  Scores: lane = key, the lane walks its key row in 8-element pieces against the R queries
+// held in LDS (fp32).  Values: lane = value dim (+ 64 c); a page's 16 tokens of that dim are two
+// 16-byte loads, 2 KiB contiguous per wave; the weights come back from LDS four at a time.
 template <int R, int NW>
 __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv,
                                                                 long q_stride, const bf16_t* __restrict__ k_cache,
                                                                 const bf16_t* __restrict__ v_cache,
                                                                 const int* __restrict__ block_tables, int bt_stride,
                                                                 const int* __restrict__ seq_lens, int Hq, int G, int dk,
-                                                                int dv, int bs, float scale, int window, int sink) {
+                                                                int dv, float scale, int window, int sink) {
+  constexpr int bs = 16;
   __shared__ __attribute__((aligned(16))) float q_s[R * kMaxDK];
+  __shared__ __attribute__((aligned(16))) float p_s[NW][R][64];
   __shared__ float ml_s[NW][R][2];
   __shared__ float acc_s[NW][R][64 * kMaxVC];
   const int b = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = seq_lens[b];
-  const int DL = dv >> 3;  // lanes that cover the value dims, 8 each
-  const int dg = lane & (DL - 1), ksub = lane / DL, KS = 64 / DL;
   bf16_t* o = out + (long)b * Hq * dv + (long)g * R * dv;
   if (n <= 0) {  // padding row of a decode bucket
     for (int c = threadIdx.x; c < R * dv; c += 64 * NW) o[c] = 0;
@@ -169,21 +169,22 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
   const int* bt = block_tables + (long)b * bt_stride;
   const int lo = window > 0 ? max(0, n - window) : 0;
   const bool first = sink && wave == 0;
-  float m[R], l[R], acc[R][8];
+  float m[R], l[R], acc[R][kMaxVC];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     m[r] = first ? 0.f : -INFINITY;
     l[r] = first ? 1.f : 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
+    for (int c = 0; c < kMaxVC; ++c) acc[r][c] = 0.f;
   }
-  const long krs = (long)G * dk, vrs = (long)G * dv;
-  for (int j0 = lo + 64 * wave; j0 < n; j0 += 64 * NW) {
+  const long krs = (long)G * dk;
+  for (int j0 = (lo & ~63) + 64 * wave; j0 < n; j0 += 64 * NW) {
     const int j = j0 + lane;
-    float sc[R], pw[R];
+    const bool valid = j >= lo && j < n;
+    float sc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) sc[r] = 0.f;
-    if (j < n) {
+    if (valid) {
       const bf16_t* kp = k_cache + ((long)bt[j / bs] * bs + j % bs) * krs + (long)g * dk;
       for (int c0 = 0; c0 < dk; c0 += 64) {  // 8 pieces of the key row in flight at a time
         uint4 kq[8];
@@ -207,48 +208,63 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
         }
       }
     }
+    // value loads of the tile's pages go out before the softmax arithmetic: 2 x 16 bytes per page and
+    // 64 dims (pages at or past the sequence's end are not touched: their weights are zero)
+    const int npg = min(4, (n - j0 + bs - 1) / bs);
+    uint4 vq[4][kMaxVC][2];
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg)
+      if (pg < npg) {
+        const long base = ((long)bt[j0 / bs + pg] * G + g) * dv;
+#pragma unroll
+        for (int c = 0; c < kMaxVC; ++c)
+          if (lane + 64 * c < dv) {
+            const uint4* vp = reinterpret_cast<const uint4*>(v_cache + (base + lane + 64 * c) * bs);
+            vq[pg][c][0] = vp[0];
+            vq[pg][c][1] = vp[1];
+          }
+      }
+    __builtin_amdgcn_wave_barrier();  // this wave's previous reads of its p_s rows come first
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float sv = j < n ? sc[r] : -INFINITY;
-      const float mt = fmaxf(m[r], wave_max(sv));  // finite: the tile holds at least key j0
-      pw[r] = j < n ? expf(sv - mt) : 0.f;
-      const float alpha = m[r] == -INFINITY ? 0.f : expf(m[r] - mt);
-      l[r] = l[r] * alpha + wave_sum(pw[r]);
+      const float sv = valid ? sc[r] : -INFINITY;
+      const float mt = fmaxf(m[r], wave_max(sv));  // the tile holds at least one live key, or m is the sink's
+      const float pw = (valid && mt != -INFINITY) ? expf(sv - mt) : 0.f;
+      const float alpha = (m[r] == -INFINITY) ? 0.f : expf(m[r] - mt);
+      l[r] = l[r] * alpha + wave_sum(pw);
       m[r] = mt;
+      p_s[wave][r][lane] = pw;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[r][i] *= alpha;
+      for (int c = 0; c < kMaxVC; ++c) acc[r][c] *= alpha;
     }
-    const int cnt = min(64, n - j0);
-    for (int i0 = 0; i0 < cnt; i0 += 4 * KS) {  // uniform trip counts: the shuffles below need every lane
-      uint4 vq[4];  // 4 value pieces in flight at a time
+    __builtin_amdgcn_wave_barrier();  // a wave's LDS instructions execute in issue order
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int jj = min(j0 + i0 + u * KS + ksub, n - 1);
-        vq[u] = *reinterpret_cast<const uint4*>(v_cache + ((long)bt[jj / bs] * bs + jj % bs) * vrs + (long)g * dv + dg * 8);
+    for (int pg = 0; pg < 4; ++pg)
+      if (pg < npg) {
+#pragma unroll
+        for (int c = 0; c < kMaxVC; ++c)
+          if (lane + 64 * c < dv) {
+            float vv[16];
+            unpack8(vq[pg][c][0], vv);
+            unpack8(vq[pg][c][1], vv + 8);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              float a = acc[r][c];
+#pragma unroll
+              for (int t4 = 0; t4 < 4; ++t4) {
+                const float4 pq = *reinterpret_cast<const float4*>(&p_s[wave][r][16 * pg + 4 * t4]);
+                a += pq.x * vv[4 * t4] + pq.y * vv[4 * t4 + 1] + pq.z * vv[4 * t4 + 2] + pq.w * vv[4 * t4 + 3];
+              }
+              acc[r][c] = a;
+            }
+          }
       }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = i0 + u * KS + ksub;
-        float vv[8];
-        unpack8(vq[u], vv);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const float pr = __shfl(pw[r], i & 63, 64);
-          const float pp = i < cnt ? pr : 0.f;
-#pragma unroll
-          for (int k = 0; k < 8; ++k) acc[r][k] += pp * vv[k];
-        }
-      }
-    }
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      float a = acc[r][k];
-      for (int off = DL; off < 64; off <<= 1) a += __shfl_xor(a, off, 64);
-      if (ksub == 0) acc_s[wave][r][dg * 8 + k] = a;
-    }
+    for (int c = 0; c < kMaxVC; ++c)
+      if (lane + 64 * c < dv) acc_s[wave][r][lane + 64 * c] = acc[r][c];
     if (lane == 0) {
       ml_s[wave][r][0] = m[r];
       ml_s[wave][r][1] = l[r];
@@ -277,7 +293,7 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
 //                             pages), B = the wave's Q rows (held in registers for the whole loop)
 //   O^T[d][q]   += V^T P^T    v_mfma_f32_16x16x16_bf16: B = the score accumulator itself (query on
 //                             the lane, 4 keys per lane: the C layout of S^T IS the B layout of P^T),
-//                             A = V^T read back transposed from an LDS copy of the 16-key V tile
+//                             A = V^T, 8-byte loads from the d-major V page (tokens contiguous)
 // With the query on the lane the running maximum, denominator and the rescale of O are lane-local
 // (two xor-shuffles per reduction).  Scores, weights and sums are fp32 (base-2 exponentials: the
 // scale carries log2 e); P is rounded to bf16 for the PV product.
@@ -285,15 +301,12 @@ template <int DK, int DV, int QT>
 __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv, long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
-    const int* __restrict__ block_tables, int bt_stride, int S, int Hq, int G, int bsh, float scale, int window,
+    const int* __restrict__ block_tables, int bt_stride, int S, int Hq, int G, float scale, int window,
     int sink) {
-  // pages hold 1 << bsh tokens; scores live in the base-2 domain (scale * log2 e folded in) so that
-  // every exponential is one v_exp_f32
-  const int bsm = (1 << bsh) - 1;
+  // pages hold 16 tokens; scores live in the base-2 domain (scale * log2 e folded in) so that every
+  // exponential is one v_exp_f32
   const float sc2 = scale * 1.44269504088896341f;
-  constexpr int VP = DV + 16;  // LDS row pitch: the 4 key rows of a fragment read land 8 banks apart
   constexpr int QB = 16 * QT;  // query rows per wave: QT tiles of 16 share every K and V^T fragment
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[16 * VP];
   int tile = blockIdx.x, s = 0, n = 0;
   for (; s < S; ++s) {  // q-blocks are numbered segment by segment
     n = cu[s + 1] - cu[s];
@@ -328,50 +341,37 @@ __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
   }
   const int lo_t = window > 0 ? max(0, p0 - window + 1) : 0, hi = p0 + nq;
   const long krs = (long)G * DK, vrs = (long)G * DV;
-  // Register double buffer: while tile j0 is computed, the K fragments and V pieces of tile j0 + 16
-  // are in flight, and the page ids of tile j0 + 32 behind them (no load waits on a load issued in
-  // the same iteration).  A lane's V pieces: piece c = lane + 64 u of the 16 x DV tile.
-  constexpr int NV = DV / 32, CPK = DV / 8;  // pieces per lane, 16-byte pieces per key
+  // Register double buffer: while tile j0 is computed, the K and V^T fragments of tile j0 + 16 are
+  // in flight, and the page id of tile j0 + 32 behind them (no load waits on a load issued in the
+  // same iteration).  A key tile is one 16-token page: its V^T fragments (4 consecutive tokens of
+  // one value dim per lane) are 8-byte loads straight from the d-major page, 512 contiguous bytes
+  // per 16 dims - no LDS, no barrier.
   const bf16_t* kbase = k_cache + (long)g * DK + 8 * quad;
-  const bf16_t* vbase = v_cache + (long)g * DV + (lane % CPK) * 8;
-  int vkey[NV];
-#pragma unroll
-  for (int u = 0; u < NV; ++u) vkey[u] = (lane + 64 * u) / CPK;
+  const bf16_t* vbase = v_cache + ((long)g * DV + c16) * 16 + 4 * quad;
   const int jfirst = lo_t & ~15;
-  auto kpage = [&](int j0) { return bt[min(j0 + c16, hi - 1) >> bsh]; };
-  auto vpage = [&](int j0, int u) { return bt[min(j0 + vkey[u], hi - 1) >> bsh]; };
-  int pk_n = kpage(jfirst), pv_n[NV];
-#pragma unroll
-  for (int u = 0; u < NV; ++u) pv_n[u] = vpage(jfirst, u);
+  int pg_n = bt[jfirst >> 4];
   bf16x8 kf_n[DK / 32];
-  uint4 vf_n[NV];
-  auto issue = [&](int j0) {  // loads of tile j0 from the page ids in pk_n / pv_n
-    const bf16_t* krow = kbase + (((long)pk_n << bsh) + (min(j0 + c16, hi - 1) & bsm)) * krs;
+  s16x4 vf_n[DV / 16];
+  auto issue = [&](int j0) {  // loads of tile j0 from the page id in pg_n
+    const bf16_t* krow = kbase + (((long)pg_n << 4) + (min(j0 + c16, hi - 1) & 15)) * krs;
 #pragma unroll
     for (int ks = 0; ks < DK / 32; ++ks) kf_n[ks] = *reinterpret_cast<const bf16x8*>(krow + 32 * ks);
+    const bf16_t* vpg = vbase + (long)pg_n * vrs * 16;
 #pragma unroll
-    for (int u = 0; u < NV; ++u)
-      vf_n[u] = *reinterpret_cast<const uint4*>(vbase + (((long)pv_n[u] << bsh) + (min(j0 + vkey[u], hi - 1) & bsm)) * vrs);
+    for (int dt = 0; dt < DV / 16; ++dt) vf_n[dt] = *reinterpret_cast<const s16x4*>(vpg + dt * 256);
   };
   issue(jfirst);
-  pk_n = kpage(jfirst + 16);
-#pragma unroll
-  for (int u = 0; u < NV; ++u) pv_n[u] = vpage(jfirst + 16, u);
+  pg_n = bt[min(jfirst + 16, hi - 1) >> 4];
   for (int j0 = jfirst; j0 < hi; j0 += 16) {
     bf16x8 kf[DK / 32];
+    s16x4 vf[DV / 16];
 #pragma unroll
     for (int ks = 0; ks < DK / 32; ++ks) kf[ks] = kf_n[ks];
-    // LDS traffic of a one-wave workgroup needs no s_barrier: a wave's LDS instructions execute in
-    // issue order, so the compiler-level barrier (no reordering across it) is all that is needed
-    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int u = 0; u < NV; ++u) *reinterpret_cast<uint4*>(&Vs[vkey[u] * VP + (lane % CPK) * 8]) = vf_n[u];
-    __builtin_amdgcn_wave_barrier();
+    for (int dt = 0; dt < DV / 16; ++dt) vf[dt] = vf_n[dt];
     if (j0 + 16 < hi) {
       issue(j0 + 16);
-      pk_n = kpage(j0 + 32);
-#pragma unroll
-      for (int u = 0; u < NV; ++u) pv_n[u] = vpage(j0 + 32, u);
+      pg_n = bt[min(j0 + 32, hi - 1) >> 4];
     }
     s16x4 pb[QT];
     float alpha[QT];
@@ -407,9 +407,7 @@ __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
     }
 #pragma unroll
     for (int dt = 0; dt < DV / 16; ++dt) {
-      s16x4 a;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] = (short)Vs[(4 * quad + i) * VP + 16 * dt + c16];
+      const s16x4 a = vf[dt];
 #pragma unroll
       for (int t = 0; t < QT; ++t) {
         if (rescale[t]) {  // wave-uniform: once the running maxima settle, most tiles skip this
@@ -442,14 +440,14 @@ using namespace k8sllm;
 extern "C" {
 
 int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float* kw, float eps, long T, int nq,
-                            int nk, int nv, void* k_cache, void* v_cache, const int* slots, int f32, hipStream_t s) {
+                            int nk, int nv, void* k_cache, void* v_cache, const int* slots, int bs, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (f32)
     hipLaunchKernelGGL(qk_norm_cache_kernel<float>, dim3(T), dim3(256), 0, s, (float*)qkv, stride, qw, kw, eps, nq, nk,
-                       nv, (float*)k_cache, (float*)v_cache, slots);
+                       nv, (float*)k_cache, (float*)v_cache, slots, bs);
   else
     hipLaunchKernelGGL(qk_norm_cache_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (bf16_t*)qkv, stride, qw, kw, eps, nq,
-                       nk, nv, (bf16_t*)k_cache, (bf16_t*)v_cache, slots);
+                       nk, nv, (bf16_t*)k_cache, (bf16_t*)v_cache, slots, bs);
   return (int)hipGetLastError();
 }
 
@@ -460,18 +458,16 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
   if (T <= 0 || S <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
   // bf16 with matrix-core head sizes and 16-byte aligned rows: the MFMA kernel
-  int bsh = 0;
-  while ((1 << bsh) < bs) ++bsh;
-  if (!f32 && mfma && (1 << bsh) == bs && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
-    // query rows per wave: 16, or 32 once the step is large enough to fill the chip that way (64
-    // shares each K / V fragment among more rows but leaves one wave per SIMD: slower); mfma = 16 /
-    // 32 / 64 forces one (tests, measurements)
-    const int qrows = mfma >= 16 ? mfma : (T * Hq >= 64 * 1024 ? 32 : 16);
+  if (!f32 && mfma && bs == 16 && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
+    // query rows per wave: 16 (measured at 8192 rows x 16 heads, window 1024: 342 us; 32 rows share
+    // each K / V^T fragment between two row tiles but run at lower occupancy: 382 us; 64: 379 us);
+    // mfma = 16 / 32 / 64 forces one (tests, measurements)
+    const int qrows = mfma >= 16 ? mfma : 16;
     const dim3 grid((unsigned)(T / qrows + S), (unsigned)Hq);
 #define K8SLLM_WP(DK, DV, QT)                                                                                          \
   hipLaunchKernelGGL((window_prefill_mfma_kernel<DK, DV, QT>), grid, dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,  \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, block_tables, bt_stride, S, Hq, \
-                     G, bsh, scale, window, sink)
+                     G, scale, window, sink)
 #define K8SLLM_WPQ(DK, DV)                                       \
   if (qrows == 64) K8SLLM_WP(DK, DV, 4);                         \
   else if (qrows == 32) K8SLLM_WP(DK, DV, 2);                    \
@@ -501,14 +497,13 @@ int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const voi
                             int dv, int bs, float scale, int window, int sink, int f32, int vec, hipStream_t s) {
   if (B <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
-  const int R = Hq / G, DL = dv / 8;
-  if (!f32 && vec && dk % 8 == 0 && dv % 8 == 0 && DL >= 1 && DL <= 64 && (DL & (DL - 1)) == 0 && q_stride % 8 == 0 &&
-      (R == 1 || R == 2 || R == 4 || R == 8)) {
+  const int R = Hq / G;
+  if (!f32 && vec && bs == 16 && dk % 8 == 0 && q_stride % 8 == 0 && (R == 1 || R == 2 || R == 4 || R == 8)) {
 #define K8SLLM_WD(RR)                                                                                                  \
   hipLaunchKernelGGL((window_decode_vec_kernel<RR, (RR == 8 ? 4 : 8)>), dim3(B, G), dim3(RR == 8 ? 256 : 512), 0, s,     \
                      (bf16_t*)out, (const bf16_t*)qkv,                                                                  \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_stride, seq_lens, Hq, G, \
-                     dk, dv, bs, scale, window, sink)
+                     dk, dv, scale, window, sink)
     if (R == 1) K8SLLM_WD(1);
     else if (R == 2) K8SLLM_WD(2);
     else if (R == 4) K8SLLM_WD(4);

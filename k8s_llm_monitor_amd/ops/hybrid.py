@@ -12,7 +12,9 @@ Conventions.  ``T`` rows are the step's tokens, all sequences concatenated; a *s
 sequence's rows of this step (a decode token is a segment of one row).  ``seg_cu`` [R+1] are the
 segments' row offsets, ``seg_ctx`` [R] the tokens each sequence already holds in its cache /
 state (0 = the sequence starts here, its state is taken as zero), ``seg_slot`` [R] its state slot
-(< 0: a padding row, skipped).  Paged caches are ``[blocks, block_size, heads * dim]``.
+(< 0: a padding row, skipped).  Paged caches: keys ``[blocks, block_size, heads * dim]`` (a token's
+keys contiguous), values ``[blocks, heads, vdim, block_size]`` (a value dim's tokens contiguous - the
+direction the PV products read along).
 """
 from __future__ import annotations
 
@@ -109,7 +111,8 @@ def qk_norm_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: fl
             ok = slot_mapping >= 0
             s = slot_mapping[ok].long()
             k_cache.view(-1, nk)[s] = qkv[ok, nq:nq + nk]
-            v_cache.view(-1, Hkv * dv)[s] = qkv[ok, nq + nk:]
+            bs = k_cache.shape[1]
+            v_cache.view(-1, Hkv * dv, bs)[s // bs, :, s % bs] = qkv[ok, nq + nk:]
         return
     native().qk_norm_cache(qkv, qw, kw, float(eps), Hq, Hkv, dk, dv, k_cache, v_cache, slot_mapping)
 
@@ -135,8 +138,8 @@ def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: 
     keys): row r of segment s at position p = ctx[s] + r sees positions max(0, p - window + 1) .. p
     (``window`` 0: all of 0 .. p).  ``sink``: the softmax denominator has one more term exp(0) that
     carries no value.  Scores and weights are fp32.  Returns [T, Hq*dv].  GPU, bf16, head sizes
-    64 / 128: the matrix-core kernel, 16 query rows per wave or 32 in large steps (``mfma`` 0: the
-    any-size wave-per-row kernel; 16 / 32 / 64: that many rows per wave whatever the step's size)."""
+    64 / 128: the matrix-core kernel, 16 query rows per wave (``mfma`` 0: the any-size wave-per-row
+    kernel; 16 / 32 / 64: that many rows per wave)."""
     T = qkv.shape[0]
     if not qkv.is_cuda:
         out = torch.empty(T, Hq * dv, dtype=qkv.dtype)
@@ -146,7 +149,7 @@ def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: 
             n_all = ctxl[s] + cul[s + 1] - cul[s]
             bt = block_tables[s, : (n_all + bs - 1) // bs].long()
             ks = k_cache[bt].reshape(-1, Hkv, dk)[:n_all].float()
-            vs = v_cache[bt].reshape(-1, Hkv, dv)[:n_all].float()
+            vs = v_cache[bt].permute(0, 3, 1, 2).reshape(-1, Hkv, dv)[:n_all].float()
             for r in range(cul[s], cul[s + 1]):
                 p = ctxl[s] + r - cul[s]
                 lo = max(0, p - window + 1) if window > 0 else 0
@@ -174,7 +177,7 @@ def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: t
             lo = max(0, n - window) if window > 0 else 0
             bt = block_tables[b, : (n + bs - 1) // bs].long()
             ks = k_cache[bt].reshape(-1, Hkv, dk)[lo:n].float()
-            vs = v_cache[bt].reshape(-1, Hkv, dv)[lo:n].float()
+            vs = v_cache[bt].permute(0, 3, 1, 2).reshape(-1, Hkv, dv)[lo:n].float()
             out[b] = _attend(qkv[b, : Hq * dk].float().view(Hq, dk), ks, vs, scale, sink).reshape(-1).to(qkv.dtype)
         return out
     out = torch.empty(B, Hq * dv, dtype=qkv.dtype, device=qkv.device)

@@ -64,7 +64,7 @@ def _paged(g, dt, lens, Hq, G, dk, dv, nb=40, bs=16, shuffle=True):
     perm = torch.randperm(nb, generator=g).tolist() if shuffle else list(range(nb))
     W = max((n + bs - 1) // bs for n in lens)
     bt = torch.zeros(len(lens), W, dtype=torch.int32)
-    kc, vc = _r(g, nb, bs, G * dk, dt=dt), _r(g, nb, bs, G * dv, dt=dt)
+    kc, vc = _r(g, nb, bs, G * dk, dt=dt), _r(g, nb, G, dv, bs, dt=dt)
     for s, n in enumerate(lens):
         for j in range((n + bs - 1) // bs):
             bt[s, j] = perm.pop()
@@ -101,7 +101,7 @@ def test_qk_norm_cache(dt):
     qkv = _r(g, T, Hq * dk + G * (dk + dv), dt=dt)
     qw, kw = _r(g, Hq * dk, s=0.3) + 1, _r(g, G * dk, s=0.3) + 1
     slots = _i32([17, 3, -1, 40, 41, 0])
-    kc, vc = torch.zeros(4, 16, G * dk, dtype=dt), torch.zeros(4, 16, G * dv, dtype=dt)
+    kc, vc = torch.zeros(4, 16, G * dk, dtype=dt), torch.zeros(4, G, dv, 16, dtype=dt)
     a_c, a_g = qkv.clone(), qkv.clone().cuda()
     kg, vg = kc.clone().cuda(), vc.clone().cuda()
     H.qk_norm_cache(a_c, qw, kw, 1e-5, Hq, G, dk, dv, kc, vc, slots)
@@ -203,7 +203,7 @@ def test_window_prefill_mfma_sees_exactly_the_window():
     kc, vc, bt = _paged(g, dt, [n], Hq, G, dk, dv)
     far = 33
     vc.mul_(0.2)
-    vc.view(-1, dv)[int(bt[0, far // 16]) * 16 + far % 16] = 100.0
+    vc[int(bt[0, far // 16]), :, :, far % 16] = 100.0
     qkv = _r(g, n, Hq * dk + G * (dk + dv), dt=dt)
     a = (Hq, G, dk, dv, 0.01, window, True)
     dev = [t.cuda() for t in (qkv, kc, vc, _i32([0, n]), _i32([0]), bt)]
@@ -213,7 +213,8 @@ def test_window_prefill_mfma_sees_exactly_the_window():
         assert seen.tolist() == [far <= r < far + window for r in range(n)]
 
 
-@pytest.mark.parametrize("dk,dv,Hq,G", [(64, 64, 4, 2), (128, 128, 8, 1), (24, 16, 2, 2), (32, 256, 4, 4), (128, 64, 4, 1)])
+@pytest.mark.parametrize("dk,dv,Hq,G", [(64, 64, 4, 2), (128, 128, 8, 1), (24, 16, 2, 2), (32, 256, 4, 4), (128, 64, 4, 1),
+                                        (48, 40, 6, 3), (16, 200, 2, 1)])
 @pytest.mark.parametrize("window", [7, 64, 100, 0])
 def test_window_decode_vec(dk, dv, Hq, G, window):
     g = _g(10)
