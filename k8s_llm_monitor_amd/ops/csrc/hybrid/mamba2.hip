@@ -13,6 +13,20 @@ namespace k8sllm {
 
 constexpr int kMaxTaps = 16;
 
+// Sum over groups of CH consecutive lanes (CH a power of two <= 32, groups aligned); lane 0 of each
+// group holds the group's total afterwards (every lane of the group does, up to CH = 16).  Row-local
+// DPP adds (one VALU instruction each, no LDS crossbar): quads by quad_perm, then the row's halves
+// and the row by the mirror controls, which pair equal partial sums.
+template <int CH>
+__device__ __forceinline__ float group_sum(float v) {
+  if (CH >= 2) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+  if (CH >= 4) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+  if (CH >= 8) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+  if (CH >= 16) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
+  if (CH >= 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void conv_silu_kernel(T* __restrict__ out, const T* __restrict__ proj, long stride,
                                                         int col0, int C, const float* __restrict__ cw,
@@ -256,17 +270,30 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ 
   for (int i = 0; i < 8; ++i) S[i] = (carried && live && n0 + i < N) ? sp[(long)(n0 + i) * P] : 0.f;
   const float A = expf(a_log[h]), Dh = d_skip[h], bias = dt_bias[h];
   const int boff = n0 + (n0 >> 6) * 4;
+  // a thread stages the same elements of every tile: their token, LDS offset and offset from the
+  // tile's first row are computed once (the division by N is ~40 instructions)
+  constexpr int NB = (TB * 8 * CH + 255) / 256;
+  int st_tt[NB], st_lds[NB], st_glb[NB];
+#pragma unroll
+  for (int u = 0; u < NB; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    const int tt = i / N, n = i - tt * N;
+    st_tt[u] = tt;  // >= TB: beyond the tile
+    st_lds[u] = tt * ROW + n + (n >> 6) * 4;
+    st_glb[u] = tt * C + inner + g * N + n;
+  }
+  const int cgap = G * N;
+  float* yp = y + (long)t0 * inner + (long)h * P + p;  // this lane's output column, advanced per tile
   for (int tb = t0; tb < t1; tb += TB) {
     const int nt = min(TB, t1 - tb);
     __syncthreads();  // the previous tile is consumed (and the zero fill is done)
-#pragma unroll 8
-    for (int i = threadIdx.x; i < nt * N; i += 256) {  // unrolled: the independent loads go out together
-      const int tt = i / N, n = i - tt * N;
-      const T* row = xbc + (long)(tb + tt) * C + inner + (long)g * N + n;
-      const int off = n + (n >> 6) * 4;
-      Bs[tt][off] = ldf(row);
-      Cs[tt][off] = ldf(row + (long)G * N);
-    }
+    const T* tile = xbc + (long)tb * C;
+#pragma unroll
+    for (int u = 0; u < NB; ++u)  // unrolled: the independent loads go out together
+      if (st_tt[u] < nt) {
+        (&Bs[0][0])[st_lds[u]] = ldf(tile + st_glb[u]);
+        (&Cs[0][0])[st_lds[u]] = ldf(tile + st_glb[u] + cgap);
+      }
     for (int i = threadIdx.x; i < nt * PB; i += 256) {
       const int tt = i / PB, pp = i % PB;
       const int pg = blockIdx.z * PB + pp;
@@ -297,10 +324,10 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(float* __restrict__ 
       S[7] = dA * S[7] + dtx * b1.w;
       float acc = S[0] * c0.x + S[1] * c0.y + S[2] * c0.z + S[3] * c0.w + S[4] * c1.x + S[5] * c1.y + S[6] * c1.z +
                   S[7] * c1.w;
-#pragma unroll
-      for (int o = 1; o < CH; o <<= 1) acc += __shfl_xor(acc, o, 64);
-      if (live && chunk == 0) y[(long)(tb + tt) * inner + (long)h * P + p] = acc + Dh * x;
+      acc = group_sum<CH>(acc);
+      if (live && chunk == 0) yp[(long)tt * inner] = acc + Dh * x;
     }
+    yp += (long)TB * inner;
   }
   if (live) {
 #pragma unroll

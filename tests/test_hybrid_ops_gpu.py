@@ -132,7 +132,8 @@ def test_conv_silu_with_state(dt, taps, C, col0, pad):
 
 
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("nh,P,N,G", [(4, 24, 12, 2), (2, 80, 40, 1), (3, 16, 130, 3)])
+@pytest.mark.parametrize("nh,P,N,G", [(4, 24, 12, 2), (2, 80, 40, 1), (3, 16, 130, 3), (2, 20, 24, 2), (2, 40, 100, 1),
+                                      (1, 8, 8, 1)])  # 2, 8, 32, 4, 16 lanes per value of p; state 8: the decode mapping only
 def test_ssm_scan_with_state(dt, nh, P, N, G):
     g = _g(6)
     new, ctx, slot = [6, 1, 3, 40, 2], [0, 9, 2, 0, 1], [1, 3, 0, 2, -1]
