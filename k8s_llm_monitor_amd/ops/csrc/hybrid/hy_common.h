@@ -41,6 +41,41 @@ __device__ __forceinline__ void load8_any(const void* p, int dt, long i, float* 
   else load8(reinterpret_cast<const bf16_t*>(p) + i, f);
 }
 
+// Wave-wide butterflies without the LDS crossbar: quads and rows by DPP (quad_perm, the row's mirror
+// controls pair equal partial results), rows 0/1 and 2/3 by v_permlane16_swap, the halves by
+// v_permlane32_swap.  Every lane ends with the result.
+#define K8SLLM_DPP(v, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true))
+__device__ __forceinline__ float xor16_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor16_max(float x) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_sum_f(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor32_max_f(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += K8SLLM_DPP(v, 0xB1);
+  v += K8SLLM_DPP(v, 0x4E);
+  v += K8SLLM_DPP(v, 0x141);
+  v += K8SLLM_DPP(v, 0x140);
+  return xor32_sum_f(xor16_sum(v));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, K8SLLM_DPP(v, 0xB1));
+  v = fmaxf(v, K8SLLM_DPP(v, 0x4E));
+  v = fmaxf(v, K8SLLM_DPP(v, 0x141));
+  v = fmaxf(v, K8SLLM_DPP(v, 0x140));
+  return xor32_max_f(xor16_max(v));
+}
+
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
 
 // the segment that holds row r: largest s with cu[s] <= r (cu has S + 1 entries, cu[0] = 0)

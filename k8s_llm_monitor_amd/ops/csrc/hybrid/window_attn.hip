@@ -68,10 +68,10 @@ __device__ __forceinline__ void attend_wave(T* __restrict__ out_row, const T* __
       for (int c = 0; c < dk; ++c) a += q_s[c] * ldf(kp + c);
       s = a;
     }
-    const float mt = fmaxf(m, wave_max(s));
+    const float mt = fmaxf(m, wave_max_dpp(s));
     const float p = j < hi ? expf(s - mt) : 0.f;
     const float alpha = expf(m - mt);  // m = -inf only before the first key (no sink): exp(-inf) = 0
-    l = l * alpha + wave_sum(p);
+    l = l * alpha + wave_sum_dpp(p);
     m = mt;
     __syncthreads();  // the previous tile's reads of p_s are done
     p_s[lane] = p;
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
 // R = Hq / G query heads of that kv head, so every cached key and value is read once.  The waves take
 // the window's 64-key tiles (aligned to 64, i.e. four whole pages) in turn and their partial (maximum,
 // denominator, output) triples are merged through LDS at the end; only wave 0 starts from the sink's
-// (0, 1).  Scores: lane = key, the lane walks its key row in 8-element pieces against the R queries
+// (0, 1); scores carry log2 e so that every exponential is one v_exp_f32.  Scores: lane = key, the lane walks its key row in 8-element pieces against the R queries
 // held in LDS (fp32).  Values: lane = value dim (+ 64 c); a page's 16 tokens of that dim are two
 // 16-byte loads, 2 KiB contiguous per wave; the weights come back from LDS four at a time.
 template <int R, int NW>
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
     return;
   }
   const bf16_t* q = qkv + (long)b * q_stride + (long)g * R * dk;
-  for (int c = threadIdx.x; c < R * dk; c += 64 * NW) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * scale;
+  for (int c = threadIdx.x; c < R * dk; c += 64 * NW) q_s[(c / dk) * kMaxDK + c % dk] = bf2f(q[c]) * (scale * 1.44269504088896341f);  // base-2 scores
   __syncthreads();
   const int* bt = block_tables + (long)b * bt_stride;
   const int lo = window > 0 ? max(0, n - window) : 0;
@@ -228,10 +228,10 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float sv = valid ? sc[r] : -INFINITY;
-      const float mt = fmaxf(m[r], wave_max(sv));  // the tile holds at least one live key, or m is the sink's
-      const float pw = (valid && mt != -INFINITY) ? expf(sv - mt) : 0.f;
-      const float alpha = (m[r] == -INFINITY) ? 0.f : expf(m[r] - mt);
-      l[r] = l[r] * alpha + wave_sum(pw);
+      const float mt = fmaxf(m[r], wave_max_dpp(sv));  // the tile holds at least one live key, or m is the sink's
+      const float pw = (valid && mt != -INFINITY) ? __builtin_amdgcn_exp2f(sv - mt) : 0.f;
+      const float alpha = (m[r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[r] - mt);
+      l[r] = l[r] * alpha + wave_sum_dpp(pw);
       m[r] = mt;
       p_s[wave][r][lane] = pw;
 #pragma unroll
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
     float L = 0.f, val = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const float f = ml_s[w][r][0] == -INFINITY ? 0.f : expf(ml_s[w][r][0] - M);
+      const float f = ml_s[w][r][0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml_s[w][r][0] - M);
       L += ml_s[w][r][1] * f;
       val += acc_s[w][r][dcol] * f;
     }
@@ -388,19 +388,17 @@ __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
         sv[i] = (q_live[t] && j >= my_lo[t] && j <= my_p[t]) ? sacc[i] * sc2 : -INFINITY;
         tmax = fmaxf(tmax, sv[i]);
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      tmax = xor32_max_f(xor16_max(tmax));
       const float mn = fmaxf(m[t], tmax);
-      alpha[t] = m[t] == -INFINITY ? 0.f : exp2f(m[t] - mn);
+      alpha[t] = m[t] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[t] - mn);
       float ps = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = sv[i] == -INFINITY ? 0.f : exp2f(sv[i] - mn);
+        const float pv = sv[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sv[i] - mn);
         ps += pv;
         pb[t][i] = (short)f2bf(pv);
       }
-      ps += __shfl_xor(ps, 16, 64);
-      ps += __shfl_xor(ps, 32, 64);
+      ps = xor32_sum_f(xor16_sum(ps));
       l[t] = l[t] * alpha[t] + ps;
       m[t] = mn;
       rescale[t] = __any(alpha[t] != 1.f);
@@ -459,10 +457,9 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
   // bf16 with matrix-core head sizes and 16-byte aligned rows: the MFMA kernel
   if (!f32 && mfma && bs == 16 && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
-    // query rows per wave: 16 (measured at 8192 rows x 16 heads, window 1024: 342 us; 32 rows share
-    // each K / V^T fragment between two row tiles but run at lower occupancy: 382 us; 64: 379 us);
-    // mfma = 16 / 32 / 64 forces one (tests, measurements)
-    const int qrows = mfma >= 16 ? mfma : 16;
+    // query rows per wave: 32 once the step is large enough to fill the chip that way (two row tiles
+    // share every K / V^T fragment), else 16; mfma = 16 / 32 / 64 forces one (tests, measurements)
+    const int qrows = mfma >= 16 ? mfma : (T * Hq >= 64 * 1024 ? 32 : 16);
     const dim3 grid((unsigned)(T / qrows + S), (unsigned)Hq);
 #define K8SLLM_WP(DK, DV, QT)                                                                                          \
   hipLaunchKernelGGL((window_prefill_mfma_kernel<DK, DV, QT>), grid, dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,  \

@@ -138,8 +138,8 @@ def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: 
     keys): row r of segment s at position p = ctx[s] + r sees positions max(0, p - window + 1) .. p
     (``window`` 0: all of 0 .. p).  ``sink``: the softmax denominator has one more term exp(0) that
     carries no value.  Scores and weights are fp32.  Returns [T, Hq*dv].  GPU, bf16, head sizes
-    64 / 128: the matrix-core kernel, 16 query rows per wave (``mfma`` 0: the any-size wave-per-row
-    kernel; 16 / 32 / 64: that many rows per wave)."""
+    64 / 128: the matrix-core kernel, 16 query rows per wave or 32 in large steps (``mfma`` 0: the
+    any-size wave-per-row kernel; 16 / 32 / 64: that many rows per wave)."""
     T = qkv.shape[0]
     if not qkv.is_cuda:
         out = torch.empty(T, Hq * dv, dtype=qkv.dtype)
