@@ -215,7 +215,7 @@ def test_window_prefill_mfma_sees_exactly_the_window():
 
 
 @pytest.mark.parametrize("dk,dv,Hq,G", [(64, 64, 4, 2), (128, 128, 8, 1), (24, 16, 2, 2), (32, 256, 4, 4), (128, 64, 4, 1),
-                                        (48, 40, 6, 3), (16, 200, 2, 1)])
+                                        (56, 40, 6, 3), (16, 200, 2, 1)])
 @pytest.mark.parametrize("window", [7, 64, 100, 0])
 def test_window_decode_vec(dk, dv, Hq, G, window):
     g = _g(10)
