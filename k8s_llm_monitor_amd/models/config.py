@@ -145,14 +145,22 @@ def get_config(name: str) -> ModelConfig:
 
 @dataclass(frozen=True)
 class MoESpec:
-    """Routed feed-forward: ``experts`` SwiGLU experts of width ``ff`` of which each token takes
-    ``top`` (weights = softmax over the chosen router logits), plus an optional shared expert of
-    width ``shared_ff`` scaled by a per-token sigmoid gate (0 = none)."""
+    """Routed feed-forward: ``experts`` experts of width ``ff`` of which each token takes ``top``,
+    plus an optional shared expert of width ``shared_ff`` (0 = none).  How the router weighs the
+    chosen experts, the experts' form and the shared expert's gate belong to the design
+    (DESIGN_TRAITS ``ffn``)."""
 
     experts: int
     top: int
     ff: int
     shared_ff: int = 0
+
+
+@dataclass(frozen=True)
+class DenseSpec:
+    """Plain feed-forward of width ``ff`` (up-projection, activation, down-projection)."""
+
+    ff: int
 
 
 @dataclass(frozen=True)
@@ -163,7 +171,7 @@ class LayerSpec:
 
     kind: str
     mixer: tuple
-    mlp: Optional[MoESpec] = None
+    mlp: Optional[object] = None  # MoESpec, DenseSpec or None
 
     @property
     def m(self) -> dict:
@@ -195,7 +203,11 @@ class HybridConfig:
 
     @property
     def is_moe(self) -> bool:
-        return any(s.mlp is not None for s in self.layers)
+        return any(isinstance(s.mlp, MoESpec) for s in self.layers)
+
+    @property
+    def traits(self) -> dict:
+        return DESIGN_TRAITS[self.arch]
 
     def runs(self) -> list:
         """Execution order as (layer index, pass number or -1, first layer of its pass)."""
@@ -212,6 +224,29 @@ class HybridConfig:
         return dataclasses.replace(self, **kw)
 
 
+# What a layer-list design fixes for all of its models (sizes and per-layer constants come from
+# the model's config.json):
+#   block          "parallel": one norm feeds mixer and feed-forward, both added to the stream;
+#                  "sequential": x += mixer(norm1(x)), then x += ff(norm2(x))
+#   one_plus_norm  RMSNorm weights are stored around zero and applied as 1 + w
+#   learned_pos    a table of absolute positions is added to the token embedding
+#   token_shift    what a mixer reads is moved towards the previous token's (per-channel weights
+#                  ``l<i>.shift``); the previous token's rows are per-sequence state
+#   depth_average  the input of layer i + 1 is a learned combination (``l<i>.dwa``) of the embedding
+#                  output and the results of layers 0 .. i
+#   ffn            the feed-forward family: "swiglu_topk" (gated experts, biased router, softmax over
+#                  the chosen logits, sigmoid-gated shared expert) or "plain_softmax" (ungated
+#                  experts with erf-GELU, softmax over all logits and the chosen probabilities
+#                  used as they are, ungated shared expert, dense layers with xIELU)
+#   max_position   positions a model accepts when its config.json does not say
+DESIGN_TRAITS = {
+    "dunesun": dict(block="parallel", one_plus_norm=True, learned_pos=True, token_shift=False,
+                    depth_average=False, ffn="swiglu_topk", max_position=2048),
+    "kisutar": dict(block="sequential", one_plus_norm=False, learned_pos=False, token_shift=True,
+                    depth_average=True, ffn="plain_softmax", max_position=1 << 17),
+}
+
+
 def _flat(d: dict, prefix: str = "") -> list:
     out = []
     for k, v in d.items():
@@ -225,27 +260,34 @@ def _flat(d: dict, prefix: str = "") -> list:
 def hybrid_config_from_dict(c: dict, name: Optional[str] = None) -> HybridConfig:
     """A :class:`HybridConfig` from a layer-list ``config.json``: ``architecture``, ``vocab``,
     ``width``, ``max_positions``, ``norm.eps``, ``logit_scale``, ``loop`` {start, stop, times} and
-    ``layers`` [{type, mixer {...}, mlp {kind, expert.ff, router.experts, router.top, shared.ff} |
-    null}].  Nested mixer keys are flattened with dots (``mask.size``)."""
+    ``layers`` [{type, mixer {...}, mlp {kind: moe, expert.ff, router.experts, router.top, shared.ff}
+    | {kind: dense, ff} | null}].  Nested mixer keys are flattened with dots (``mask.size``)."""
+    arch = str(c["architecture"]).lower()
+    if arch not in DESIGN_TRAITS:
+        raise ValueError(f"unknown architecture {c['architecture']!r} (known: {sorted(DESIGN_TRAITS)})")
     layers = []
     for spec in c["layers"]:
         ml = spec.get("mlp")
         moe = None
         if ml is not None:
-            if ml.get("kind", "moe") != "moe":
-                raise ValueError(f"unsupported feed-forward kind {ml.get('kind')!r}")
-            sh = ml.get("shared")
-            moe = MoESpec(experts=int(ml["router"]["experts"]), top=int(ml["router"]["top"]),
-                          ff=int(ml["expert"]["ff"]), shared_ff=int(sh["ff"]) if sh else 0)
+            kind = ml.get("kind", "moe")
+            if kind == "moe":
+                sh = ml.get("shared")
+                moe = MoESpec(experts=int(ml["router"]["experts"]), top=int(ml["router"]["top"]),
+                              ff=int(ml["expert"]["ff"]), shared_ff=int(sh["ff"]) if sh else 0)
+            elif kind == "dense":
+                moe = DenseSpec(ff=int(ml["ff"]))
+            else:
+                raise ValueError(f"unsupported feed-forward kind {kind!r}")
         layers.append(LayerSpec(kind=spec["type"], mixer=tuple(sorted(_flat(spec.get("mixer") or {}))), mlp=moe))
     lp = c.get("loop")
     loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else None
     if loop and not (0 <= loop[0] < loop[1] <= len(layers) and loop[2] >= 1):
         raise ValueError(f"bad loop {lp!r} for {len(layers)} layers")
     V = int(c["vocab"])
-    return HybridConfig(name=name or str(c.get("architecture", "hybrid")).lower(),
-                        arch=str(c["architecture"]).lower(), vocab_size=V, d_model=int(c["width"]),
-                        layers=tuple(layers), max_position=int(c.get("max_positions", 2048)),
+    return HybridConfig(name=name or arch, arch=arch, vocab_size=V, d_model=int(c["width"]),
+                        layers=tuple(layers),
+                        max_position=int(c.get("max_positions", DESIGN_TRAITS[arch]["max_position"])),
                         norm_eps=float(c["norm"]["eps"]), logit_scale=float(c.get("logit_scale", 1.0)), loop=loop,
                         bos_id=int(c.get("bos_id", min(1, V - 1))), eos_ids=tuple(c.get("eos_ids", (min(2, V - 1),))))
 
@@ -265,7 +307,9 @@ def hybrid_config_to_dict(c: HybridConfig) -> dict:
     layers = []
     for s in c.layers:
         ml = None
-        if s.mlp is not None:
+        if isinstance(s.mlp, DenseSpec):
+            ml = {"kind": "dense", "ff": s.mlp.ff}
+        elif s.mlp is not None:
             ml = {"kind": "moe", "expert": {"ff": s.mlp.ff}, "router": {"experts": s.mlp.experts, "top": s.mlp.top},
                   "shared": {"ff": s.mlp.shared_ff} if s.mlp.shared_ff else None}
         layers.append({"type": s.kind, "mixer": nest(s.mixer), "mlp": ml})
@@ -287,7 +331,15 @@ def _ssm(heads, vdim, state, groups, conv, norm_groups):
                                              "conv": conv, "norm_groups": norm_groups}.items())))
 
 
-def _with_mlp(s: LayerSpec, m: Optional[MoESpec]) -> LayerSpec:
+def _latent(heads, dim, rot_dim, vdim, q_rank, kv_rank, window, scale, base=10000.0, kv_from=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+         "mask.size": window, "scale": scale, "rot.base": base, "rot.dims": rot_dim}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return LayerSpec("latent_attention", tuple(sorted(m.items())))
+
+
+def _with_mlp(s: LayerSpec, m) -> LayerSpec:
     return dataclasses.replace(s, mlp=m)
 
 
@@ -300,3 +352,13 @@ DUNESUN_TINY = _reg(HybridConfig(
             _with_mlp(_ssm(2, 64, 32, 1, 3, 1), None),
             _with_mlp(_attn(2, 2, 64, 64, 8, 0.125), MoESpec(6, 3, 32, 64))),
     max_position=1024, loop=(1, 3, 2), logit_scale=1.5, bos_id=1, eos_ids=(2,)))
+
+# Small Kisutar-design model for CPU tests and GPU smoke runs (random weights): latent attention in
+# every layer, the last two reading layer 1's compressed keys, dense / routed / no feed-forward.
+KISUTAR_TINY = _reg(HybridConfig(
+    name="kisutar-tiny", arch="kisutar", vocab_size=384, d_model=96,
+    layers=(_with_mlp(_latent(4, 24, 8, 16, 40, 32, 20, 0.18), DenseSpec(160)),
+            _with_mlp(_latent(2, 32, 16, 24, 48, 40, 12, 0.15), MoESpec(6, 2, 48, 64)),
+            _with_mlp(_latent(4, 16, 16, 32, 32, 40, 28, 0.2, kv_from=1), None),
+            _with_mlp(_latent(2, 24, 16, 24, 24, 40, 9, 0.17, kv_from=1), MoESpec(4, 3, 32, 0))),
+    max_position=4096, norm_eps=1e-6, bos_id=1, eos_ids=(2,)))

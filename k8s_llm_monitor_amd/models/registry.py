@@ -12,14 +12,14 @@ from typing import Optional, Union
 import torch
 
 from .checkpoint import SafetensorsDir, config_from_hf, load_checkpoint
-from .config import HybridConfig, ModelConfig, hybrid_config_from_dict
+from .config import DESIGN_TRAITS, HybridConfig, ModelConfig, hybrid_config_from_dict
 from .hybrid import HybridLM
 from .llama import CausalLM
 
 # config.arch -> model class
-MODEL_CLASSES = {"llama": CausalLM, "gpt2": CausalLM, "dunesun": HybridLM}
+MODEL_CLASSES = {"llama": CausalLM, "gpt2": CausalLM, "dunesun": HybridLM, "kisutar": HybridLM}
 # layer-list designs by the ``architecture`` value of their config.json (lower case)
-LAYER_LIST_ARCHS = {"dunesun"}
+LAYER_LIST_ARCHS = set(DESIGN_TRAITS)
 
 
 def config_from_dir(path: Union[str, Path], name: Optional[str] = None):

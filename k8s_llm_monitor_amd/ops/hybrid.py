@@ -1,7 +1,9 @@
 """Operators of the layer-list (hybrid) decoders: fp32 residual stream with one-plus RMSNorm,
 windowed attention with a softmax sink over a paged cache, the Mamba-2 recurrence with its short
 convolution and per-sequence state slots, and routed experts with a biased fp32 router and a
-gated shared expert.
+gated shared expert; and, for the sequential-block designs, the token-shifted norm, the depth
+average of layer results, latent (low-rank compressed) attention with rotary positions and learned
+per-head sinks, and ungated experts with a softmax-over-all router.
 
 GPU tensors run the gfx950 kernels of ``_k8sllm_hybrid`` (``ops/csrc/hybrid``; built by
 ``python -m k8s_llm_monitor_amd.ops.build --only hybrid``) for bfloat16 and float32 activations
@@ -57,15 +59,22 @@ def _silu(z: torch.Tensor) -> torch.Tensor:
 # ---------------------------------------------------------------- residual stream / norms
 
 def embed_pos(ids: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, pos: Optional[torch.Tensor],
-              src: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None) -> torch.Tensor:
+              src: Optional[torch.Tensor] = None, prev: Optional[torch.Tensor] = None,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 rows ``embed[id] + pos[position]`` (``pos`` None: no learned positions).  ``src`` /
-    ``prev`` (pipelined decode): row i takes token ``prev[src[i]]`` where ``src[i] >= 0``."""
+    ``prev`` (pipelined decode): row i takes token ``prev[src[i]]`` where ``src[i] >= 0``.
+    ``out``: a contiguous fp32 [T, d] buffer to fill."""
     if not embed.is_cuda:
         if src is not None:
             ids = torch.where(src >= 0, prev.index_select(0, src.clamp(min=0).long()), ids)
         x = embed[ids.long()].float()
-        return x + pos[positions.long()].float() if pos is not None else x
-    out = torch.empty(ids.numel(), embed.shape[1], dtype=torch.float32, device=embed.device)
+        x = x + pos[positions.long()].float() if pos is not None else x
+        if out is not None:
+            out.copy_(x)
+            return out
+        return x
+    if out is None:
+        out = torch.empty(ids.numel(), embed.shape[1], dtype=torch.float32, device=embed.device)
     native().embed_pos(out, ids, positions, embed, pos, src, prev)
     return out
 
@@ -88,6 +97,77 @@ def add_norm(residual: torch.Tensor, addends: tuple, vec: Optional[torch.Tensor]
     out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
     a = list(addends) + [None] * (3 - len(addends))
     native().add_norm(out, residual, a[0], a[1], a[2], vec, w, float(eps), bool(one_plus))
+    return out
+
+
+def norm_shift(residual: torch.Tensor, addends: tuple, w: torch.Tensor, eps: float, one_plus: bool,
+               mu: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor,
+               seg_slot: torch.Tensor, out_dtype: torch.dtype, advance: bool = True) -> torch.Tensor:
+    """Token-shifted norm.  ``residual`` (fp32 [T, d], updated in place) += ``addends``; with
+    ``h[t]`` the RMSNorm of row t times ``w`` (fp32), returns ``h[t] + (h[t-1] - h[t]) * mu`` in
+    ``out_dtype``, where the row before a segment's first comes from ``state[slot]`` ([slots, d]
+    fp32; zeros where seg_ctx is 0).  ``advance``: ``state[slot]`` then takes the segment's last
+    ``h`` (unshifted).  GPU: the state of segments longer than one row is advanced by a second
+    small launch, after every row has read the old state."""
+    if not residual.is_cuda:
+        for a in addends:
+            residual += a.float()
+        h = residual * torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps)
+        wf = w.float()
+        h = h * (1.0 + wf if one_plus else wf)
+        prev = torch.zeros_like(h)
+        prev[1:] = h[:-1]
+        cul = seg_cu.tolist()
+        for s, (c0, slot) in enumerate(zip(seg_ctx.tolist(), seg_slot.tolist())):
+            a, b = cul[s], cul[s + 1]
+            if b <= a:
+                continue
+            prev[a] = state[slot] if (c0 > 0 and slot >= 0) else 0.0
+            if advance and slot >= 0:
+                state[slot] = h[b - 1]
+        return (h + (prev - h) * mu.float()).to(out_dtype)
+    assert len(addends) <= 2
+    out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    a = list(addends) + [None] * (2 - len(addends))
+    native().norm_shift(out, residual, a[0], a[1], w, float(eps), bool(one_plus), mu, state, seg_cu, seg_ctx, seg_slot,
+                        bool(advance))
+    return out
+
+
+def depth_mix(stack: torch.Tensor, n: int, addend: Optional[torch.Tensor], coef: torch.Tensor) -> torch.Tensor:
+    """Depth-weighted average.  ``stack`` [L, T, d] fp32 holds the embedding output and the layer
+    results so far in entries 0 .. n (entry n is the newest, still missing ``addend``):
+    ``stack[n] += addend``, then ``stack[n + 1] = sum_j coef[j] * stack[j]`` over j = 0 .. n
+    (``coef`` [n + 1] fp32).  Returns ``stack[n + 1]``, the next layer's input."""
+    if not stack.is_cuda:
+        if addend is not None:
+            stack[n] += addend.float()
+        stack[n + 1] = torch.einsum("j,jtd->td", coef.float(), stack[: n + 1])
+        return stack[n + 1]
+    native().depth_mix(stack, int(n), addend, coef)
+    return stack[n + 1]
+
+
+ACTS = {"gelu": 0, "gelu_tanh": 1, "xielu": 2}
+
+
+def activation(x: torch.Tensor, kind: str, a: float = 0.0, b: float = 0.0) -> torch.Tensor:
+    """Elementwise on [T, f] rows, evaluated in fp32: ``gelu`` (erf form), ``gelu_tanh``, or
+    ``xielu`` with the two positive constants ``a``, ``b``:  z > 0: a z^2 + z / 2;  z <= 0:
+    b (exp(z) - 1 - z) + z / 2."""
+    if not x.is_cuda:
+        z = x.float()
+        if kind == "gelu":
+            y = F.gelu(z)
+        elif kind == "gelu_tanh":
+            y = F.gelu(z, approximate="tanh")
+        elif kind == "xielu":
+            y = torch.where(z > 0, a * z * z + 0.5 * z, b * (torch.expm1(z.clamp(max=0.0)) - z) + 0.5 * z)
+        else:
+            raise ValueError(kind)
+        return y.to(x.dtype)
+    out = torch.empty_like(x)
+    native().activation(out, x, ACTS[kind], float(a), float(b))
     return out
 
 
@@ -117,27 +197,32 @@ def qk_norm_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: fl
     native().qk_norm_cache(qkv, qw, kw, float(eps), Hq, Hkv, dk, dv, k_cache, v_cache, slot_mapping)
 
 
-def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, sink: bool) -> torch.Tensor:
-    """q [H, dk], k [n, G, dk], v [n, G, dv] (fp32) -> [H, dv]."""
+def _attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, sink: bool,
+            sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q [H, dk], k [n, G, dk], v [n, G, dv] (fp32) -> [H, dv].  ``sinks`` [H]: the sink's logit per
+    head (absent: 0)."""
     H, G = q.shape[0], k.shape[1]
     kk = k.repeat_interleave(H // G, dim=1)
     vv = v.repeat_interleave(H // G, dim=1)
     s = torch.einsum("hd,nhd->hn", q, kk) * scale
     m = s.max(-1, keepdim=True).values
+    z = sinks.float().view(H, 1) if sinks is not None else torch.zeros(H, 1)
     if sink:
-        m = m.clamp(min=0.0)
+        m = torch.maximum(m, z)
     e = torch.exp(s - m)
-    den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sink else 0.0)
+    den = e.sum(-1, keepdim=True) + (torch.exp(z - m) if sink else 0.0)
     return torch.einsum("hn,nhd->hd", e / den, vv)
 
 
 def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu: torch.Tensor,
                              ctx: torch.Tensor, block_tables: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int,
-                             scale: float, window: int, sink: bool, mfma: int = 1) -> torch.Tensor:
+                             scale: float, window: int, sink: bool, mfma: int = 1,
+                             sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the step's prompt chunks over the paged cache (which already holds their own
     keys): row r of segment s at position p = ctx[s] + r sees positions max(0, p - window + 1) .. p
-    (``window`` 0: all of 0 .. p).  ``sink``: the softmax denominator has one more term exp(0) that
-    carries no value.  Scores and weights are fp32.  Returns [T, Hq*dv].  GPU, bf16, head sizes
+    (``window`` 0: all of 0 .. p).  ``sink``: the softmax denominator has one more term that carries
+    no value - exp(0), or exp(sinks[h]) for head h where ``sinks`` [Hq] fp32 is given (a learned,
+    unscaled logit).  Scores and weights are fp32.  Returns [T, Hq*dv].  GPU, bf16, head sizes
     64 / 128: the matrix-core kernel, 16 query rows per wave or 32 in large steps (``mfma`` 0: the
     any-size wave-per-row kernel; 16 / 32 / 64: that many rows per wave)."""
     T = qkv.shape[0]
@@ -153,18 +238,19 @@ def window_attention_prefill(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: 
             for r in range(cul[s], cul[s + 1]):
                 p = ctxl[s] + r - cul[s]
                 lo = max(0, p - window + 1) if window > 0 else 0
-                o = _attend(qkv[r, : Hq * dk].float().view(Hq, dk), ks[lo:p + 1], vs[lo:p + 1], scale, sink)
+                o = _attend(qkv[r, : Hq * dk].float().view(Hq, dk), ks[lo:p + 1], vs[lo:p + 1], scale, sink, sinks)
                 out[r] = o.reshape(-1).to(qkv.dtype)
         return out
     out = torch.empty(T, Hq * dv, dtype=qkv.dtype, device=qkv.device)
     native().window_attention_prefill(out, qkv, k_cache, v_cache, cu, ctx, block_tables, Hq, Hkv, dk, dv, float(scale),
-                                      int(window), bool(sink), int(mfma))
+                                      int(window), bool(sink), sinks, int(mfma))
     return out
 
 
 def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             block_tables: torch.Tensor, seq_lens: torch.Tensor, Hq: int, Hkv: int, dk: int, dv: int,
-                            scale: float, window: int, sink: bool, vec: bool = True) -> torch.Tensor:
+                            scale: float, window: int, sink: bool, vec: bool = True,
+                            sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One query per sequence (its newest token, already in the cache) over the last ``window``
     cached positions; ``seq_lens`` count that token (0: a padding row, output zero)."""
     B = qkv.shape[0]
@@ -178,11 +264,71 @@ def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: t
             bt = block_tables[b, : (n + bs - 1) // bs].long()
             ks = k_cache[bt].reshape(-1, Hkv, dk)[lo:n].float()
             vs = v_cache[bt].permute(0, 3, 1, 2).reshape(-1, Hkv, dv)[lo:n].float()
-            out[b] = _attend(qkv[b, : Hq * dk].float().view(Hq, dk), ks, vs, scale, sink).reshape(-1).to(qkv.dtype)
+            out[b] = _attend(qkv[b, : Hq * dk].float().view(Hq, dk), ks, vs, scale, sink,
+                             sinks).reshape(-1).to(qkv.dtype)
         return out
     out = torch.empty(B, Hq * dv, dtype=qkv.dtype, device=qkv.device)
     native().window_attention_decode(out, qkv, k_cache, v_cache, block_tables, seq_lens, Hq, Hkv, dk, dv, float(scale),
-                                     int(window), bool(sink), bool(vec))
+                                     int(window), bool(sink), sinks, bool(vec))
+    return out
+
+
+# ---------------------------------------------------------------- latent attention
+
+def _rotate_half(v: torch.Tensor, pos: torch.Tensor, base: float, dims: int) -> torch.Tensor:
+    """v [T, ..., n] fp32: the first ``dims`` entries of the last axis turn in pairs (i, i + dims/2) by
+    the angle pos * base^(-2i/dims) (angles in fp32); the rest pass."""
+    half = dims // 2
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                  -2.0 * torch.arange(half, dtype=torch.float64) / dims).float().to(v.device)
+    a = pos.float().view(-1, *([1] * (v.dim() - 1))) * f
+    c, s = torch.cos(a), torch.sin(a)
+    u, x = v[..., :half], v[..., half:dims]
+    return torch.cat([u * c - x * s, x * c + u * s, v[..., dims:]], -1)
+
+
+def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw: torch.Tensor,
+                kw: Optional[torch.Tensor], eps: float, positions: torch.Tensor, base: float, dims: int,
+                k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                slot_mapping: Optional[torch.Tensor]) -> None:
+    """In place on the fused down-projections [T, q_rank | kv_rank | rot_dim] (or [T, q_rank] for a
+    layer that reads another layer's cache): the query latent is RMS-normed (weight ``qw``); the
+    key/value latent is RMS-normed (weight ``kw``) and the shared key part behind it is rotated by
+    its position; both go to the pages at ``slot_mapping`` - the key page row is [latent | rotated
+    part], the value page holds the latent once more, dim-major."""
+    T = proj.shape[0]
+    if not proj.is_cuda:
+        q = proj[:, :q_rank].float()
+        proj[:, :q_rank] = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw.float()).to(proj.dtype)
+        if k_cache is None:
+            return
+        c = proj[:, q_rank:q_rank + kv_rank].float()
+        c = (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kw.float()).to(proj.dtype)
+        kr = _rotate_half(proj[:, q_rank + kv_rank:].float(), positions, base, dims).to(proj.dtype)
+        proj[:, q_rank:q_rank + kv_rank] = c
+        proj[:, q_rank + kv_rank:] = kr
+        ok = slot_mapping >= 0
+        s = slot_mapping[ok].long()
+        bs = k_cache.shape[1]
+        k_cache.view(-1, kv_rank + rot_dim)[s] = proj[ok, q_rank:]
+        v_cache.view(-1, kv_rank, bs)[s // bs, :, s % bs] = c[ok]
+        return
+    native().latent_prep(proj, int(q_rank), int(kv_rank), int(rot_dim), qw, kw, float(eps), positions, float(base),
+                         int(dims), k_cache, v_cache, slot_mapping)
+
+
+def latent_queries(q: torch.Tensor, q_lat: torch.Tensor, H: int, dim: int, rot_dim: int, positions: torch.Tensor,
+                   base: float, dims: int) -> torch.Tensor:
+    """The queries against the latent cache: per head [q_lat | rotated part], [T, H * (R + rot_dim)].
+    ``q`` [T, H * (dim + rot_dim)] are the up-projected queries (their last ``rot_dim`` entries per
+    head are rotated by the position) and ``q_lat`` [H, T, R] the unrotated parts already
+    multiplied into the latent space."""
+    T, R = q.shape[0], q_lat.shape[2]
+    if not q.is_cuda:
+        qr = _rotate_half(q.view(T, H, dim + rot_dim)[..., dim:].float(), positions, base, dims).to(q.dtype)
+        return torch.cat([q_lat.transpose(0, 1), qr], -1).reshape(T, H * (R + rot_dim))
+    out = torch.empty(T, H * (R + rot_dim), dtype=q.dtype, device=q.device)
+    native().latent_queries(out, q, q_lat, int(H), int(dim), int(rot_dim), positions, float(base), int(dims))
     return out
 
 
@@ -279,9 +425,11 @@ def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col: int, w: torch.T
 
 # ---------------------------------------------------------------- routed experts
 
-def moe_router(h: torch.Tensor, wr: torch.Tensor, bias: torch.Tensor, E: int, K: int) -> tuple:
-    """fp32 router: logits = ``wr[:E] h + bias[:E]``, the ``K`` largest are chosen and weighted by
-    the softmax over the chosen logits only.  ``wr`` may hold one more row (E + 1 in all): then
+def moe_router(h: torch.Tensor, wr: torch.Tensor, bias: Optional[torch.Tensor], E: int, K: int,
+               over_all: bool = False) -> tuple:
+    """fp32 router: logits = ``wr[:E] h + bias[:E]`` (``bias`` None: none), the ``K`` largest are
+    chosen and weighted by the softmax over the chosen logits only - or, ``over_all``, by their
+    probabilities in the softmax over all E logits, as they are.  ``wr`` may hold one more row (E + 1 in all): then
     ``gate = sigmoid(wr[E] h)`` per token is returned too (the shared expert's gate).
     Returns (ids [T, K] int32, weights [T, K] fp32, gate [T] fp32 or None)."""
     T = h.shape[0]
@@ -289,12 +437,15 @@ def moe_router(h: torch.Tensor, wr: torch.Tensor, bias: torch.Tensor, E: int, K:
     if not h.is_cuda:
         lg = h.float() @ wr.float().t()
         gate = torch.sigmoid(lg[:, E]) if has_gate else None
-        top, idx = torch.topk(lg[:, :E] + bias.float()[:E], K, dim=-1)
+        z = lg[:, :E] + bias.float()[:E] if bias is not None else lg[:, :E]
+        top, idx = torch.topk(z, K, dim=-1)
+        if over_all:
+            return idx.to(torch.int32), torch.softmax(z, -1).gather(1, idx), gate
         return idx.to(torch.int32), torch.softmax(top, -1), gate
     ids = torch.empty(T, K, dtype=torch.int32, device=h.device)
     wts = torch.empty(T, K, dtype=torch.float32, device=h.device)
     gate = torch.empty(T, dtype=torch.float32, device=h.device) if has_gate else None
-    native().moe_router(ids, wts, gate, h, wr, bias, E, K)
+    native().moe_router(ids, wts, gate, h, wr, bias, E, K, bool(over_all))
     return ids, wts, gate
 
 
@@ -305,11 +456,12 @@ TILE_MIN_ROWS = 1024
 
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
                 shared: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, il: bool = False,
-                mfma: bool = True) -> torch.Tensor:
+                mfma: bool = True, act: str = "swiglu") -> torch.Tensor:
     """Sum over each token's chosen experts of ``wts * down_e(silu(gate_e h) * up_e h)`` with
     ``w13`` [E, 2*ff, d] (gate rows then up rows; ``il``: interleaved per 128 rows as [64 gate |
     64 up], ops.interleave_gate_up) and ``w2`` [E, d, ff], plus ``gate * shared`` (the shared
-    expert's output [T, d] and its per-token gate).  fp32 [T, d].
+    expert's output [T, d] and its per-token gate; ``gate`` None: 1).  ``act`` "gelu": ungated
+    experts ``down_e(gelu(up_e h))`` with ``w13`` [E, ff, d].  fp32 [T, d].
 
     GPU: the (token, slot) pairs are counting-sorted by expert on the device and both projections
     run as ONE grouped launch each over the sorted rows (SwiGLU in the first epilogue); no host
@@ -329,10 +481,13 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
                 if il:
                     we = we.view(ff // 64, 2, 64, d).permute(1, 0, 2, 3).reshape(2 * ff, d)
                 gu = (hf[rows] @ we.t()).to(h.dtype).float()
-                act = (_silu(gu[:, :ff]) * gu[:, ff:]).to(h.dtype).float()
-                out.index_add_(0, rows, (act @ w2[e].float().t()).to(h.dtype).float() * wts[rows, slot].unsqueeze(-1))
+                if act == "gelu":
+                    a = F.gelu(gu).to(h.dtype).float()
+                else:
+                    a = (_silu(gu[:, :ff]) * gu[:, ff:]).to(h.dtype).float()
+                out.index_add_(0, rows, (a @ w2[e].float().t()).to(h.dtype).float() * wts[rows, slot].unsqueeze(-1))
         if shared is not None:
-            out += shared.float() * gate.unsqueeze(-1)
+            out += shared.float() * gate.unsqueeze(-1) if gate is not None else shared.float()
         return out
     ext = native()
     n = T * K
@@ -340,17 +495,18 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
     sorted_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     inv_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     ext.moe_align(ids, E, offsets, sorted_idx, inv_idx)
+    code = {"swiglu": 1, "gelu": 2}[act]
     if il and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16:
         from .. import ops  # the Mixtral path's kernels (_k8sllm_ops)
 
         xs = ops.gather_rows(h, sorted_idx, K)
-        act = ops.moe_grouped_gemm(xs, w13, offsets, swiglu=True, zero_fill=False)
-        ys = ops.moe_grouped_gemm(act, w2, offsets, zero_fill=False)
+        a = ops.moe_grouped_gemm(xs, w13, offsets, swiglu=True, zero_fill=False)
+        ys = ops.moe_grouped_gemm(a, w2, offsets, zero_fill=False)
     else:
-        act = torch.empty(n, ff, dtype=h.dtype, device=h.device)
-        ext.grouped_gemm(act, h, w13, offsets, sorted_idx, K, True, il, mfma)
+        a = torch.empty(n, ff, dtype=h.dtype, device=h.device)
+        ext.grouped_gemm(a, h, w13, offsets, sorted_idx, K, code, il, mfma)
         ys = torch.empty(n, d, dtype=h.dtype, device=h.device)
-        ext.grouped_gemm(ys, act, w2, offsets, None, 1, False, False, mfma)
+        ext.grouped_gemm(ys, a, w2, offsets, None, 1, 0, False, mfma)
     out = torch.empty(T, d, dtype=torch.float32, device=h.device)
     ext.moe_combine(out, ys, inv_idx, wts, shared, gate)
     return out
