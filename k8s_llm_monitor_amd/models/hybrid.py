@@ -204,6 +204,7 @@ class LatentAttention:
         self.w_uk = p.get(prefix + "uk", (H * dn, R), 1.0 / math.sqrt(R))  # viewed [H, dn, R]
         self.w_uv = p.get(prefix + "uv", (H * dv, R), 1.0 / math.sqrt(R))  # viewed [H, dv, R]
         self.sinks = p.get(prefix + "sink", (H,), 1.0, small=True)
+        self.freq = hops.rotary_freq(self.base, self.rdims, p.device)
         self.wo = p.get(prefix + "o", (d, H * dv), 1.0 / math.sqrt(H * dv))
 
     def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
@@ -221,12 +222,12 @@ class LatentAttention:
         down = F.linear(h, self.w_down)
         kc, vc = cache["k"], cache["v"]
         own = self.kv_from is None
-        hops.latent_prep(down, Q, R, dr, self.qn, self.kn, self.eps, meta.positions, self.base, self.rdims,
+        hops.latent_prep(down, Q, R, dr, self.qn, self.kn, self.eps, meta.positions, self.freq,
                          kc if own else None, vc if own else None, meta.slot_mapping if own else None)
         q = F.linear(down[:, :Q], self.w_uq)
         # the per-head key expansion moved to the query: q_lat[h] = q_unrotated[h] @ W_uk[h]  ([H, T, R])
         q_lat = torch.bmm(q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1), self.w_uk.view(H, dn, R))
-        qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.base, self.rdims)
+        qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.freq)
         args = (H, 1, R + dr, R, self.scale, self.window, True)
         if not meta.is_prefill:
             o = hops.window_attention_decode(qa, kc, vc, meta.block_tables, meta.seq_lens, *args, vec=bool(self.fast),
@@ -496,7 +497,7 @@ class HybridLM:
                 x += self.loop_step[t]
             if self.shifted:
                 h = hops.norm_shift(x, pending, self.norms[li], c.norm_eps, self.one_plus, self.shifts[li],
-                                    caches[r]["shift"], *seg, self.dtype)
+                                    caches[r]["shift"], *seg, self.dtype, multi=meta.is_prefill)
             else:
                 h = hops.add_norm(x, pending, None, self.norms[li], c.norm_eps, self.one_plus, self.dtype)
             pending = (self.mixers[li].forward(h, meta, caches[self.kv_run[r]]),)

@@ -18,11 +18,12 @@ int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float
                             int nk, int nv, void* k_cache, void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
 int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                              const int* cu, const int* ctx, const int* block_tables, int bt_stride, int S, long T,
-                             int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink, int f32,
-                             int mfma, hipStream_t s);
+                             int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink,
+                             const float* sinks, int f32, int mfma, hipStream_t s);
 int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                             const int* block_tables, int bt_stride, const int* seq_lens, int B, int Hq, int G, int dk,
-                            int dv, int bs, float scale, int window, int sink, int f32, int vec, hipStream_t s);
+                            int dv, int bs, float scale, int window, int sink, const float* sinks, int f32, int vec,
+                            hipStream_t s);
 int k8sllm_hy_conv_silu(void* out, const void* proj, long stride, int col0, int C, const float* cw, const float* cb,
                         int taps, void* state, const int* cu, const int* ctx, const int* slot, int S, long T, int f32,
                         hipStream_t s);
@@ -30,12 +31,23 @@ int k8sllm_hy_ssm_scan(float* y, const void* xbc, const void* proj, long p_strid
                        const float* a_log, const float* d_skip, float* state, const int* cu, const int* ctx,
                        const int* slot, int S, long T, int nh, int P, int N, int G, int f32, int mode, hipStream_t s);
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
-                     const float* bias, int E, int K, int rows_w, int f32, hipStream_t s);
+                     const float* bias, int E, int K, int rows_w, int over_all, int f32, hipStream_t s);
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
-                           int E, long rows, int N, int Kd, long w_es, int swiglu, int il, int f32, int mfma,
+                           int E, long rows, int N, int Kd, long w_es, int act, int il, int f32, int mfma,
                            hipStream_t s);
 int k8sllm_hy_combine(float* out, const void* ys, const int* inv, const float* wts, const void* shared,
                       const float* gate, long T, int K, int d, int f32, hipStream_t s);
+int k8sllm_hy_norm_shift(void* out, const float* x, const float* w, const float* mu, float* state, const int* cu,
+                         const int* ctx, const int* slot, int S, long rows, int d, float eps, int one_plus,
+                         int advance, int multi, int f32, hipStream_t s);
+int k8sllm_hy_depth_mix(float* stack, long plane, int n, const void* addend, int adt, const float* coef,
+                        hipStream_t s);
+int k8sllm_hy_activation(void* out, const void* x, long n, int kind, float a, float b, int f32, hipStream_t s);
+int k8sllm_hy_latent_prep(void* proj, long stride, long T, int Q, int R, int dr, const float* qw, const float* kw,
+                          float eps, const int* positions, const float* freq, int nf, void* k_cache, void* v_cache,
+                          const int* slots, int bs, int f32, hipStream_t s);
+int k8sllm_hy_latent_queries(void* out, const void* q, long q_stride, const void* q_lat, long T, int H, int dn, int dr,
+                             int R, const int* positions, const float* freq, int nf, int f32, hipStream_t s);
 int k8sllm_moe_align(const int* topk_ids, long n, int E, int* expert_offsets, int* sorted_idx, int* inv_idx,
                      hipStream_t s);
 }
@@ -155,6 +167,14 @@ void vpages(const Tensor& c, const Tensor& k, int f, int64_t G, int64_t dv) {
               "v_cache must be [blocks, kv_heads, vdim, block]");
 }
 
+// learned sink logits, one per query head (absent: every sink's logit is 0)
+const float* sink_ptr(const OptT& sinks, int64_t Hq) {
+  if (!sinks.has_value()) return nullptr;
+  f32c(*sinks, "sinks");
+  TORCH_CHECK(sinks->numel() == Hq, "sinks [Hq]");
+  return sinks->data_ptr<float>();
+}
+
 void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int64_t G, int64_t dk, int64_t dv,
                    OptT k_cache, OptT v_cache, OptT slots) {
   const int f = act(qkv, "qkv");
@@ -182,7 +202,7 @@ void qk_norm_cache(Tensor qkv, Tensor qw, Tensor kw, double eps, int64_t Hq, int
 
 void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor cu, Tensor ctx,
                               Tensor block_tables, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
-                              int64_t window, bool sink, int64_t mfma) {
+                              int64_t window, bool sink, OptT sinks, int64_t mfma) {
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
@@ -200,13 +220,14 @@ void window_attention_prefill(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_c
   check(k8sllm_hy_window_prefill(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                  cu.data_ptr<int>(), ctx.data_ptr<int>(), block_tables.data_ptr<int>(),
                                  (int)block_tables.stride(0), (int)S, T, (int)Hq, (int)G, (int)dk, (int)dv,
-                                 (int)k_cache.size(1), (float)scale, (int)window, sink, f, (int)mfma, cur()),
+                                 (int)k_cache.size(1), (float)scale, (int)window, sink, sink_ptr(sinks, Hq), f,
+                                 (int)mfma, cur()),
         "window_attention_prefill");
 }
 
 void window_attention_decode(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_cache, Tensor block_tables,
                              Tensor seq_lens, int64_t Hq, int64_t G, int64_t dk, int64_t dv, double scale,
-                             int64_t window, bool sink, bool vec) {
+                             int64_t window, bool sink, OptT sinks, bool vec) {
   const int f = act(qkv, "qkv");
   same(out, f, "out");
   pages(k_cache, f, G * dk, "k_cache");
@@ -223,7 +244,7 @@ void window_attention_decode(Tensor out, Tensor qkv, Tensor k_cache, Tensor v_ca
   check(k8sllm_hy_window_decode(out.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                 block_tables.data_ptr<int>(), (int)block_tables.stride(0), seq_lens.data_ptr<int>(),
                                 (int)B, (int)Hq, (int)G, (int)dk, (int)dv, (int)k_cache.size(1), (float)scale,
-                                (int)window, sink, f, vec, cur()),
+                                (int)window, sink, sink_ptr(sinks, Hq), f, vec, cur()),
         "window_attention_decode");
 }
 
@@ -279,16 +300,20 @@ void ssm_scan(Tensor y, Tensor xbc, Tensor proj, int64_t dt_col, Tensor dt_bias,
         "ssm_scan");
 }
 
-void moe_router(Tensor ids, Tensor wts, OptT gate, Tensor h, Tensor wr, Tensor bias, int64_t E, int64_t K) {
+void moe_router(Tensor ids, Tensor wts, OptT gate, Tensor h, Tensor wr, OptT bias, int64_t E, int64_t K,
+                bool over_all) {
   const int f = act(h, "h");
   i32c(ids, "ids");
   f32c(wts, "wts");
   f32c(wr, "router weight");
-  f32c(bias, "router bias");
+  if (bias.has_value()) {
+    f32c(*bias, "router bias");
+    TORCH_CHECK(bias->numel() >= E, "router bias [E]");
+  }
   const int64_t T = h.size(0), d = h.size(1);
   TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && wr.dim() == 2 && wr.size(1) == d, "router: h [T, d], wr [E(+1), d]");
   TORCH_CHECK(wr.size(0) == E || wr.size(0) == E + 1, "router rows");
-  TORCH_CHECK(bias.numel() >= E && ids.numel() == T * K && wts.numel() == T * K, "router: bias / outputs");
+  TORCH_CHECK(ids.numel() == T * K && wts.numel() == T * K, "router: outputs");
   TORCH_CHECK(E <= 256 && K >= 1 && K <= 16 && K <= E, "router: up to 256 experts, top 16");
   float* gp = nullptr;
   if (gate.has_value()) {
@@ -297,7 +322,8 @@ void moe_router(Tensor ids, Tensor wts, OptT gate, Tensor h, Tensor wr, Tensor b
     gp = gate->data_ptr<float>();
   }
   check(k8sllm_hy_router(ids.data_ptr<int>(), wts.data_ptr<float>(), gp, h.data_ptr(), T, (int)d, wr.data_ptr<float>(),
-                         bias.data_ptr<float>(), (int)E, (int)K, (int)wr.size(0), f, cur()),
+                         bias.has_value() ? bias->data_ptr<float>() : nullptr, (int)E, (int)K, (int)wr.size(0), over_all,
+                         f, cur()),
         "moe_router");
 }
 
@@ -314,8 +340,11 @@ void moe_align(Tensor ids, int64_t E, Tensor offsets, Tensor sorted_idx, Tensor 
 }
 
 // y [rows, N] = W[e] a over expert-sorted rows; sorted_idx given: a's row of sorted row r is sorted_idx[r] / div
-void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx, int64_t div, bool swiglu, bool il,
+// act_code: 0 none, 1 SwiGLU (w = [gate rows ; up rows]), 2 erf GELU
+void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx, int64_t div, int64_t act_code, bool il,
                   bool mfma) {
+  TORCH_CHECK(act_code >= 0 && act_code <= 2, "grouped_gemm: activation code");
+  const bool swiglu = act_code == 1;
   const int f = act(a, "a");
   same(y, f, "y");
   same(w, f, "w");
@@ -334,7 +363,7 @@ void grouped_gemm(Tensor y, Tensor a, Tensor w, Tensor offsets, OptT sorted_idx,
     TORCH_CHECK(a.size(0) == rows, "grouped_gemm: a rows");
   }
   check(k8sllm_hy_grouped_gemm(y.data_ptr(), a.data_ptr(), w.data_ptr(), offsets.data_ptr<int>(), sp, (int)div, (int)E,
-                               rows, (int)N, (int)Kd, w.size(1) * Kd, swiglu, il, f, mfma, cur()),
+                               rows, (int)N, (int)Kd, w.size(1) * Kd, (int)act_code, il, f, mfma, cur()),
         "grouped_gemm");
 }
 
@@ -351,15 +380,106 @@ void moe_combine(Tensor out, Tensor ys, Tensor inv, Tensor wts, OptT shared, Opt
   const float* gp = nullptr;
   if (shared.has_value()) {
     same(*shared, f, "shared");
-    TORCH_CHECK(gate.has_value() && shared->is_contiguous() && shared->numel() == T * d, "shared [T, d] with its gate");
-    f32c(*gate, "gate");
-    TORCH_CHECK(gate->numel() == T, "gate [T]");
+    TORCH_CHECK(shared->is_contiguous() && shared->numel() == T * d, "shared [T, d]");
     sh = shared->data_ptr();
-    gp = gate->data_ptr<float>();
+    if (gate.has_value()) {
+      f32c(*gate, "gate");
+      TORCH_CHECK(gate->numel() == T, "gate [T]");
+      gp = gate->data_ptr<float>();
+    }
   }
   check(k8sllm_hy_combine(out.data_ptr<float>(), ys.data_ptr(), inv.data_ptr<int>(), wts.data_ptr<float>(), sh, gp, T,
                           (int)K, (int)d, f, cur()),
         "moe_combine");
+}
+
+void norm_shift(Tensor out, Tensor x, Tensor w, double eps, bool one_plus, Tensor mu, Tensor state, Tensor cu, Tensor ctx,
+                Tensor slot, bool advance, bool multi) {
+  const int f = act(out, "out");
+  f32c(x, "residual");
+  f32c(w, "w");
+  f32c(mu, "shift");
+  f32c(state, "shift state");
+  segs(cu, ctx, slot);
+  TORCH_CHECK(x.dim() == 2 && out.is_contiguous() && out.numel() == x.numel(), "norm_shift: out shape");
+  const int64_t rows = x.size(0), d = x.size(1);
+  TORCH_CHECK(w.numel() == d && mu.numel() == d && state.dim() == 2 && state.size(1) == d, "norm_shift: w, shift [d], state [slots, d]");
+  check(k8sllm_hy_norm_shift(out.data_ptr(), x.data_ptr<float>(), w.data_ptr<float>(), mu.data_ptr<float>(),
+                             state.data_ptr<float>(), cu.data_ptr<int>(), ctx.data_ptr<int>(), slot.data_ptr<int>(),
+                             (int)ctx.numel(), rows, (int)d, (float)eps, one_plus, advance, multi, f, cur()),
+        "norm_shift");
+}
+
+void depth_mix(Tensor stack, int64_t n, OptT addend, Tensor coef) {
+  f32c(stack, "stack");
+  f32c(coef, "coef");
+  TORCH_CHECK(stack.dim() == 3 && n >= 0 && n + 1 < stack.size(0) && coef.numel() == n + 1 && n < 256,
+              "depth_mix: stack [L, T, d], coef [n + 1], n + 1 < L");
+  const int64_t plane = stack.size(1) * stack.size(2);
+  TORCH_CHECK(plane % 4 == 0, "depth_mix: T * d must be a multiple of 4");
+  const int adt = any_dt(addend, plane, "addend");
+  check(k8sllm_hy_depth_mix(stack.data_ptr<float>(), plane, (int)n, adt ? addend->data_ptr() : nullptr, adt,
+                            coef.data_ptr<float>(), cur()),
+        "depth_mix");
+}
+
+void activation(Tensor out, Tensor x, int64_t kind, double a, double b) {
+  const int f = act(x, "x");
+  same(out, f, "out");
+  TORCH_CHECK(x.is_contiguous() && out.is_contiguous() && out.numel() == x.numel() && kind >= 0 && kind <= 2, "activation: shapes / kind");
+  check(k8sllm_hy_activation(out.data_ptr(), x.data_ptr(), x.numel(), (int)kind, (float)a, (float)b, f, cur()), "activation");
+}
+
+void latent_prep(Tensor proj, int64_t Q, int64_t R, int64_t dr, Tensor qw, OptT kw, double eps, Tensor positions,
+                 Tensor freq, OptT k_cache, OptT v_cache, OptT slots) {
+  const int f = act(proj, "proj");
+  f32c(qw, "dq.norm");
+  f32c(freq, "freq");
+  i32c(positions, "positions");
+  const int64_t T = proj.size(0);
+  const bool own = kw.has_value();
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && proj.size(1) == (own ? Q + R + dr : Q), "proj [T, q_rank (+ kv_rank + rot)]");
+  TORCH_CHECK(qw.numel() == Q && positions.numel() >= T && 2 * freq.numel() <= dr, "latent_prep: norm weight / positions / freq");
+  void *kc = nullptr, *vc = nullptr;
+  const int* sp = nullptr;
+  const float* kwp = nullptr;
+  int bs = 16;
+  if (own) {
+    f32c(*kw, "dkv.norm");
+    TORCH_CHECK(kw->numel() == R, "dkv.norm [kv_rank]");
+    kwp = kw->data_ptr<float>();
+    if (k_cache.has_value()) {
+      TORCH_CHECK(v_cache.has_value() && slots.has_value(), "k_cache, v_cache and slot_mapping come together");
+      pages(*k_cache, f, R + dr, "k_cache");
+      vpages(*v_cache, *k_cache, f, 1, R);
+      sp = iptr(slots, "slot_mapping");
+      TORCH_CHECK(slots->numel() >= T, "slot_mapping [T]");
+      kc = k_cache->data_ptr();
+      vc = v_cache->data_ptr();
+      bs = (int)k_cache->size(1);
+    }
+  }
+  check(k8sllm_hy_latent_prep(proj.data_ptr(), proj.stride(0), T, (int)Q, (int)R, (int)dr, qw.data_ptr<float>(), kwp,
+                              (float)eps, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), kc, vc, sp,
+                              bs, f, cur()),
+        "latent_prep");
+}
+
+void latent_queries(Tensor out, Tensor q, Tensor q_lat, int64_t H, int64_t dn, int64_t dr, Tensor positions, Tensor freq) {
+  const int f = act(q, "q");
+  same(out, f, "out");
+  same(q_lat, f, "q_lat");
+  f32c(freq, "freq");
+  i32c(positions, "positions");
+  const int64_t T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * (dn + dr), "q [T, H * (dim + rot)]");
+  TORCH_CHECK(q_lat.dim() == 3 && q_lat.is_contiguous() && q_lat.size(0) == H && q_lat.size(1) == T, "q_lat [H, T, R]");
+  const int64_t R = q_lat.size(2);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * (R + dr) && positions.numel() >= T && 2 * freq.numel() <= dr,
+              "latent_queries: out / positions / freq");
+  check(k8sllm_hy_latent_queries(out.data_ptr(), q.data_ptr(), q.stride(0), q_lat.data_ptr(), T, (int)H, (int)dn, (int)dr,
+                                 (int)R, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), f, cur()),
+        "latent_queries");
 }
 
 }  // namespace
@@ -378,4 +498,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_align", &moe_align);
   m.def("grouped_gemm", &grouped_gemm);
   m.def("moe_combine", &moe_combine);
+  m.def("norm_shift", &norm_shift);
+  m.def("depth_mix", &depth_mix);
+  m.def("activation", &activation);
+  m.def("latent_prep", &latent_prep);
+  m.def("latent_queries", &latent_queries);
 }

@@ -1,11 +1,14 @@
 // Routed feed-forward of the layer-list decoders (any sizes, bf16 or fp32 activations).
-//   moe_router    fp32 logits = Wr h + b (h widened from its storage dtype), the K largest chosen
-//                 (lowest index wins a tie), weights = softmax over the chosen logits only; one
-//                 more row of Wr, if present, gives gate = sigmoid(Wr[E] h) (the shared expert's)
+//   moe_router    fp32 logits = Wr h + b (h widened from its storage dtype; b may be absent), the K
+//                 largest chosen (lowest index wins a tie), weights = softmax over the chosen logits
+//                 only, or (over_all) the chosen experts' probabilities in the softmax over all E
+//                 logits, not renormalised; one more row of Wr, if present, gives
+//                 gate = sigmoid(Wr[E] h) (the shared expert's)
 //   grouped_gemm  Y[r] = W[e(r)] A[row(r)] over expert-sorted rows r (offsets / sorted_idx from the
-//                 counting sort), the A rows gathered on load; SWIGLU: W = [gate rows ; up rows] and
-//                 Y = silu(gate) * up.  64 x 64 tiles, fp32 accumulation.
-//   moe_combine   out[t] = sum_k w[t][k] Y[inv[t*K + k]] + gate[t] * shared[t]   (fp32)
+//                 counting sort), the A rows gathered on load; ACT 1 (SwiGLU): W = [gate rows ; up
+//                 rows] and Y = silu(gate) * up; ACT 2: Y = gelu(W A) (erf form).  64 x 64 tiles, fp32
+//                 accumulation.
+//   moe_combine   out[t] = sum_k w[t][k] Y[inv[t*K + k]] + gate[t] * shared[t]   (fp32; no gate: 1)
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -20,7 +23,7 @@ template <typename T, int NACC>
 __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                         float* __restrict__ gate, const T* __restrict__ h, int d,
                                                         const float* __restrict__ wr, const float* __restrict__ bias,
-                                                        int E, int K, int rows_w) {
+                                                        int E, int K, int rows_w, int over_all) {
   __shared__ float lg[kMaxE + 1];
   __shared__ float part[4][NACC > 0 ? NACC : 1];
   const long t = blockIdx.x;
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, f
     if (threadIdx.x < rows_w) {
       const int e = threadIdx.x;
       const float a = part[0][e] + part[1][e] + part[2][e] + part[3][e];
-      lg[e] = e < E ? a + bias[e] : a;
+      lg[e] = (e < E && bias != nullptr) ? a + bias[e] : a;
     }
   } else {
     for (int e = wave; e < rows_w; e += 4) {
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, f
       float a = 0.f;
       for (int c = lane; c < d; c += 64) a += ldf(x + c) * w[c];
       a = wave_sum(a);
-      if (lane == 0) lg[e] = e < E ? a + bias[e] : a;
+      if (lane == 0) lg[e] = (e < E && bias != nullptr) ? a + bias[e] : a;
     }
   }
   __syncthreads();
@@ -93,9 +96,14 @@ __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, f
       mx = fmaxf(mx, bv);
     }
     float z = 0.f;
-    for (int k = 0; k < K; ++k) {
-      val[k] = expf(val[k] - mx);
-      z += val[k];
+    if (over_all) {  // the denominator runs over every expert (val[0] is the largest logit of all)
+      for (int e = 0; e < E; ++e) z += expf(lg[e] - mx);
+      for (int k = 0; k < K; ++k) val[k] = expf(val[k] - mx);
+    } else {
+      for (int k = 0; k < K; ++k) {
+        val[k] = expf(val[k] - mx);
+        z += val[k];
+      }
     }
     for (int k = 0; k < K; ++k) {
       ids[t * K + k] = sel[k];
@@ -107,11 +115,14 @@ __global__ __launch_bounds__(256) void hy_router_kernel(int* __restrict__ ids, f
 
 constexpr int TM = 64, TN = 64, TK = 16;
 
-template <typename T, bool SWIGLU>
+__device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+
+template <typename T, int ACT>
 __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y, const T* __restrict__ A,
                                                               const T* __restrict__ W, const int* __restrict__ offsets,
                                                               const int* __restrict__ sorted_idx, int div, int E,
                                                               int N, int Kd, long w_es, int il) {
+  constexpr bool SWIGLU = ACT == 1;
   __shared__ float As[TK][TM + 4];
   __shared__ float Ws[TK][TN + 4];
   __shared__ float Us[SWIGLU ? TK : 1][TN + 4];
@@ -189,6 +200,10 @@ __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y,
         stf(&gq, v);
         stf(&uq, accu[i][j]);
         v = silu_f(ldf(&gq)) * ldf(&uq);
+      } else if (ACT == 2) {  // the projection is rounded to the storage dtype before the activation
+        T gq;
+        stf(&gq, v);
+        v = gelu_erf_f(ldf(&gq));
       }
       stf(Y + (long)r * N + n, v);
     }
@@ -203,12 +218,13 @@ __global__ __launch_bounds__(256) void hy_grouped_gemm_kernel(T* __restrict__ Y,
 // rows per expert (decode) make this a weight-streaming kernel: many small workgroups, no LDS.
 // ``il``: the gate / up rows are interleaved per 128 rows as [64 gate | 64 up] (the prefill tile
 // GEMM's pairing), else [all gate rows ; all up rows].
-template <bool SWIGLU, int NT>
+template <int ACT, int NT>
 __global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __restrict__ Y, const bf16_t* __restrict__ A,
                                                                   const bf16_t* __restrict__ W,
                                                                   const int* __restrict__ offsets,
                                                                   const int* __restrict__ sorted_idx, int div, int E,
                                                                   int N, int Kd, long w_es, int il) {
+  constexpr bool SWIGLU = ACT == 1;
   int e = 0, tile = blockIdx.x, r0 = 0, r1 = 0;
   for (; e < E; ++e) {
     r0 = offsets[e];
@@ -257,6 +273,7 @@ __global__ __launch_bounds__(64) void hy_grouped_gemm_mfma_kernel(bf16_t* __rest
       if (r >= r1) continue;
       float v = acc[t][i];
       if (SWIGLU) v = silu_f(bf2f(f2bf(v))) * bf2f(f2bf(accu[t][i]));
+      else if (ACT == 2) v = gelu_erf_f(bf2f(f2bf(v)));
       Y[(long)r * N + n] = f2bf(v);
     }
   }
@@ -271,7 +288,7 @@ __global__ __launch_bounds__(256) void hy_combine_kernel(float* __restrict__ out
   for (int c = threadIdx.x; c < d; c += 256) {
     float a = 0.f;
     for (int k = 0; k < K; ++k) a += wts[t * K + k] * ldf(ys + (long)inv[t * K + k] * d + c);
-    if (shared != nullptr) a += gate[t] * ldf(shared + t * d + c);
+    if (shared != nullptr) a += (gate != nullptr ? gate[t] : 1.f) * ldf(shared + t * d + c);
     out[t * d + c] = a;
   }
 }
@@ -283,12 +300,12 @@ using namespace k8sllm;
 extern "C" {
 
 int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, int d, const float* wr,
-                     const float* bias, int E, int K, int rows_w, int f32, hipStream_t s) {
+                     const float* bias, int E, int K, int rows_w, int over_all, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (E > kMaxE || K > kMaxK || K > E || K < 1 || rows_w < E || rows_w > E + 1) return -1;
 #define K8SLLM_RT(T_, NACC)                                                                                       \
   hipLaunchKernelGGL((hy_router_kernel<T_, NACC>), dim3(T), dim3(256), 0, s, ids, wts, gate, (const T_*)h, d, wr, bias, \
-                     E, K, rows_w)
+                     E, K, rows_w, over_all)
   if (f32) {
     if (rows_w <= 9) K8SLLM_RT(float, 9); else if (rows_w <= 17) K8SLLM_RT(float, 17); else K8SLLM_RT(float, 0);
   } else {
@@ -300,9 +317,11 @@ int k8sllm_hy_router(int* ids, float* wts, float* gate, const void* h, long T, i
 
 // rows: the sorted rows in all (an upper bound of the row tiles is rows / 64 + E)
 int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* offsets, const int* sorted_idx, int div,
-                           int E, long rows, int N, int Kd, long w_es, int swiglu, int il, int f32, int mfma,
+                           int E, long rows, int N, int Kd, long w_es, int act, int il, int f32, int mfma,
                            hipStream_t s) {
   if (rows <= 0) return 0;
+  if (act < 0 || act > 2) return -1;
+  const bool swiglu = act == 1;
   if (il && (!swiglu || N % 64)) return -1;
   if (!f32 && mfma && Kd % 32 == 0) {
     const bool few = rows <= 512;  // a decode-sized step: one n-tile per wave
@@ -311,9 +330,11 @@ int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* off
   hipLaunchKernelGGL((hy_grouped_gemm_mfma_kernel<SW, NT>), g16, dim3(64), 0, s, (bf16_t*)Y, (const bf16_t*)A,      \
                      (const bf16_t*)W, offsets, sorted_idx, div, E, N, Kd, w_es, il)
     if (swiglu) {
-      if (few) K8SLLM_GM(true, 1); else K8SLLM_GM(true, 4);
+      if (few) K8SLLM_GM(1, 1); else K8SLLM_GM(1, 4);
+    } else if (act == 2) {
+      if (few) K8SLLM_GM(2, 1); else K8SLLM_GM(2, 4);
     } else {
-      if (few) K8SLLM_GM(false, 1); else K8SLLM_GM(false, 4);
+      if (few) K8SLLM_GM(0, 1); else K8SLLM_GM(0, 4);
     }
 #undef K8SLLM_GM
     return (int)hipGetLastError();
@@ -323,9 +344,9 @@ int k8sllm_hy_grouped_gemm(void* Y, const void* A, const void* W, const int* off
   hipLaunchKernelGGL((hy_grouped_gemm_kernel<T, SW>), grid, dim3(256), 0, s, (T*)Y, (const T*)A, (const T*)W, offsets, \
                      sorted_idx, div, E, N, Kd, w_es, il)
   if (f32) {
-    if (swiglu) K8SLLM_GG(float, true); else K8SLLM_GG(float, false);
+    if (swiglu) K8SLLM_GG(float, 1); else if (act == 2) K8SLLM_GG(float, 2); else K8SLLM_GG(float, 0);
   } else {
-    if (swiglu) K8SLLM_GG(bf16_t, true); else K8SLLM_GG(bf16_t, false);
+    if (swiglu) K8SLLM_GG(bf16_t, 1); else if (act == 2) K8SLLM_GG(bf16_t, 2); else K8SLLM_GG(bf16_t, 0);
   }
 #undef K8SLLM_GG
   return (int)hipGetLastError();

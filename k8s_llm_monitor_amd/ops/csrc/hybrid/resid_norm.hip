@@ -3,6 +3,10 @@
 //   add_norm          residual += a0 + a1 + a2 + vec;  out = residual / rms(residual) * (w | 1 + w)
 //   gated_group_norm  out = group_rms_norm(y * silu(z)) * w       (y fp32, groups of equal size)
 //   swiglu            out = silu(gu[:, :f]) * gu[:, f:]
+//   norm_shift        h[t] = x[t] / rms(x[t]) * w;  out[t] = h[t] + (h[t-1] - h[t]) * mu, the row before
+//                     a segment from the sequence's state slot; shift_state advances the slots
+//   depth_mix         stack[n] += addend;  stack[n+1] = sum_j coef[j] * stack[j], j = 0 .. n
+//   activation        erf GELU, tanh GELU or xIELU, elementwise in fp32
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -120,6 +124,121 @@ __global__ __launch_bounds__(256) void swiglu_kernel(T* __restrict__ out, const 
   stf(out + i, silu_f(ldf(gu + r * 2 * f + c)) * ldf(gu + r * 2 * f + f + c));
 }
 
+
+// Token-shifted RMSNorm, one workgroup per row.  The row also norms its predecessor (the same fp32
+// arithmetic in the same order as that row's own workgroup, so a prompt cut anywhere gives the same
+// values); a segment's first row reads the sequence's slot instead (zeros for a fresh sequence).  A
+// one-row segment writes its h to the slot right here (each thread overwrites only what it has read);
+// longer segments leave that to shift_state_kernel, launched after every row has read the old slot.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_shift_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                         const float* __restrict__ w, const float* __restrict__ mu,
+                                                         float* __restrict__ state, const int* __restrict__ cu,
+                                                         const int* __restrict__ ctx, const int* __restrict__ slot,
+                                                         int S, int d, float eps, int one_plus, int advance) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  const int s = find_segment(cu, S, (int)row);
+  const bool first = row == cu[s], single = first && cu[s + 1] - cu[s] == 1;
+  const int sl = slot[s];
+  const float* xr = x + row * d;
+  const float* xp = xr - d;
+  float ss = 0.f, sp = 0.f;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const float v = xr[c];
+    ss += v * v;
+    if (!first) {
+      const float u = xp[c];
+      sp += u * u;
+    }
+  }
+  ss = block_sum<256>(ss, red);
+  if (!first) sp = block_sum<256>(sp, red);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps), invp = 1.0f / sqrtf(sp / (float)d + eps);
+  const bool from_state = first && sl >= 0 && ctx[s] > 0;
+  float* st = sl >= 0 ? state + (long)sl * d : nullptr;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const float g = one_plus ? 1.f + w[c] : w[c];
+    const float h = xr[c] * inv * g;
+    float hp = 0.f;
+    if (!first) hp = xp[c] * invp * g;
+    else if (from_state) hp = st[c];
+    stf(out + row * d + c, h + (hp - h) * mu[c]);
+    if (advance && single && st != nullptr) st[c] = h;
+  }
+}
+
+template <int DUMMY>
+__global__ __launch_bounds__(256) void shift_state_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                          float* __restrict__ state, const int* __restrict__ cu,
+                                                          const int* __restrict__ slot, int d, float eps,
+                                                          int one_plus) {
+  __shared__ float red[4];
+  const int s = blockIdx.x;
+  const int n = cu[s + 1] - cu[s], sl = slot[s];
+  if (n < 2 || sl < 0) return;  // one-row segments were advanced by their own row
+  const float* xr = x + (long)(cu[s + 1] - 1) * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += 256) ss += xr[c] * xr[c];
+  ss = block_sum<256>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += 256) state[(long)sl * d + c] = xr[c] * inv * (one_plus ? 1.f + w[c] : w[c]);
+}
+
+constexpr int kMaxDepth = 256;
+
+// 4 consecutive elements per thread; entry n of the stack is completed with the addend on the way.
+__global__ __launch_bounds__(256) void depth_mix_kernel(float* __restrict__ stack, long plane, int n,
+                                                        const void* __restrict__ addend, int adt,
+                                                        const float* __restrict__ coef) {
+  __shared__ float cf[kMaxDepth];
+  for (int j = threadIdx.x; j <= n; j += 256) cf[j] = coef[j];
+  __syncthreads();
+  const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= plane) return;
+  float4 top = *reinterpret_cast<const float4*>(stack + (long)n * plane + i);
+  if (adt) {
+    top.x += ld_any(addend, adt, i);
+    top.y += ld_any(addend, adt, i + 1);
+    top.z += ld_any(addend, adt, i + 2);
+    top.w += ld_any(addend, adt, i + 3);
+    *reinterpret_cast<float4*>(stack + (long)n * plane + i) = top;
+  }
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int j = 0; j < n; ++j) {
+    const float4 v = *reinterpret_cast<const float4*>(stack + (long)j * plane + i);
+    const float a = cf[j];
+    acc.x += a * v.x; acc.y += a * v.y; acc.z += a * v.z; acc.w += a * v.w;
+  }
+  const float a = cf[n];
+  acc.x += a * top.x; acc.y += a * top.y; acc.z += a * top.z; acc.w += a * top.w;
+  *reinterpret_cast<float4*>(stack + (long)(n + 1) * plane + i) = acc;
+}
+
+// KIND 0: erf GELU, 1: tanh GELU, 2: xIELU (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below)
+template <int KIND>
+__device__ __forceinline__ float act_f(float z, float a, float b) {
+  if (KIND == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+  if (KIND == 1) return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+  return z > 0.f ? a * z * z + 0.5f * z : b * (expm1f(z) - z) + 0.5f * z;
+}
+
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ out, const T* __restrict__ x, long n, float a,
+                                                         float b) {
+  const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i >= n) return;
+  if (i + 8 <= n) {  // n a multiple of 8 whenever rows are: 16 / 32-byte accesses
+    float v[8];
+    load8(x + i, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = act_f<KIND>(v[k], a, b);
+    store8(out + i, v);
+    return;
+  }
+  for (long k = i; k < n; ++k) stf(out + k, act_f<KIND>(ldf(x + k), a, b));
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -173,6 +292,43 @@ int k8sllm_hy_swiglu(void* out, const void* gu, long rows, int f, int f32, hipSt
     hipLaunchKernelGGL(swiglu_kernel<float>, dim3(g), dim3(256), 0, s, (float*)out, (const float*)gu, rows, f);
   else
     hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(g), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)gu, rows, f);
+  return (int)hipGetLastError();
+}
+int k8sllm_hy_norm_shift(void* out, const float* x, const float* w, const float* mu, float* state, const int* cu,
+                         const int* ctx, const int* slot, int S, long rows, int d, float eps, int one_plus,
+                         int advance, int multi, int f32, hipStream_t s) {
+  if (rows <= 0 || S <= 0) return 0;
+  if (f32)
+    hipLaunchKernelGGL(norm_shift_kernel<float>, dim3(rows), dim3(256), 0, s, (float*)out, x, w, mu, state, cu, ctx,
+                       slot, S, d, eps, one_plus, advance);
+  else
+    hipLaunchKernelGGL(norm_shift_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, (bf16_t*)out, x, w, mu, state, cu, ctx,
+                       slot, S, d, eps, one_plus, advance);
+  if (advance && multi)
+    hipLaunchKernelGGL(shift_state_kernel<0>, dim3(S), dim3(256), 0, s, x, w, state, cu, slot, d, eps, one_plus);
+  return (int)hipGetLastError();
+}
+
+// plane = T * d (a multiple of 4)
+int k8sllm_hy_depth_mix(float* stack, long plane, int n, const void* addend, int adt, const float* coef,
+                        hipStream_t s) {
+  if (plane <= 0) return 0;
+  if (n < 0 || n >= kMaxDepth || (plane & 3)) return -1;
+  hipLaunchKernelGGL(depth_mix_kernel, dim3((unsigned)((plane / 4 + 255) / 256)), dim3(256), 0, s, stack, plane, n,
+                     addend, adt, coef);
+  return (int)hipGetLastError();
+}
+
+int k8sllm_hy_activation(void* out, const void* x, long n, int kind, float a, float b, int f32, hipStream_t s) {
+  if (n <= 0) return 0;
+  const dim3 g((unsigned)((n + 2047) / 2048));
+#define K8SLLM_ACT(T, K) hipLaunchKernelGGL((activation_kernel<T, K>), g, dim3(256), 0, s, (T*)out, (const T*)x, n, a, b)
+  if (f32) {
+    if (kind == 0) K8SLLM_ACT(float, 0); else if (kind == 1) K8SLLM_ACT(float, 1); else if (kind == 2) K8SLLM_ACT(float, 2); else return -1;
+  } else {
+    if (kind == 0) K8SLLM_ACT(bf16_t, 0); else if (kind == 1) K8SLLM_ACT(bf16_t, 1); else if (kind == 2) K8SLLM_ACT(bf16_t, 2); else return -1;
+  }
+#undef K8SLLM_ACT
   return (int)hipGetLastError();
 }
 }

@@ -5,8 +5,8 @@
 // Pages: k_cache [blocks][BS][G*dk] (a token's keys contiguous), v_cache [blocks][G][dv][BS] (a value
 // dim's BS tokens contiguous: the layout the PV products read along); a sequence's page list is a row of
 // block_tables.  Row at position p sees positions max(0, p - window + 1) .. p (window 0: 0 .. p).
-// The sink is one more softmax term with score 0 and no value: the running maximum starts at 0 and
-// the running denominator at 1.  Scores, weights and the output accumulation are fp32.
+// The sink is one more softmax term with no value and a fixed score - 0, or a learned unscaled logit
+// per query head (sinks[h]): the running maximum starts at that score and the running denominator at 1.  Scores, weights and the output accumulation are fp32.
 #include "hy_common.h"
 
 namespace k8sllm {
@@ -50,11 +50,11 @@ template <typename T>
 __device__ __forceinline__ void attend_wave(T* __restrict__ out_row, const T* __restrict__ q_row,
                                             const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                             const int* __restrict__ bt, int lo, int hi, int g, int G, int dk, int dv,
-                                            int bs, float scale, int sink, float* q_s, float* p_s) {
+                                            int bs, float scale, int sink, float sink_z, float* q_s, float* p_s) {
   const int lane = threadIdx.x & 63;
   for (int c = lane; c < dk; c += 64) q_s[c] = ldf(q_row + c) * scale;
   __syncthreads();  // one wave per workgroup: orders the LDS writes before the other lanes' reads
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float m = sink ? sink_z : -INFINITY, l = sink ? 1.f : 0.f;  // the sink: one term exp(sink_z - m)
   float acc[kMaxVC];
 #pragma unroll
   for (int c = 0; c < kMaxVC; ++c) acc[c] = 0.f;
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(64) void window_prefill_kernel(T* __restrict__ out,
                                                             const int* __restrict__ cu, const int* __restrict__ ctx,
                                                             const int* __restrict__ block_tables, int bt_stride, int S,
                                                             int Hq, int G, int dk, int dv, int bs, float scale,
-                                                            int window, int sink) {
+                                                            int window, int sink, const float* __restrict__ sinks) {
   __shared__ float q_s[kMaxDK];
   __shared__ float p_s[64];
   const int r = blockIdx.x, h = blockIdx.y;
@@ -112,7 +112,8 @@ __global__ __launch_bounds__(64) void window_prefill_kernel(T* __restrict__ out,
   const int p = ctx[s] + r - cu[s];
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
   attend_wave<T>(out + (long)r * Hq * dv + (long)h * dv, qkv + (long)r * q_stride + (long)h * dk, k_cache, v_cache,
-                 block_tables + (long)s * bt_stride, lo, p + 1, h / (Hq / G), G, dk, dv, bs, scale, sink, q_s, p_s);
+                 block_tables + (long)s * bt_stride, lo, p + 1, h / (Hq / G), G, dk, dv, bs, scale, sink,
+                 sinks != nullptr ? sinks[h] : 0.f, q_s, p_s);
 }
 
 template <typename T>
@@ -121,7 +122,8 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
                                                            const T* __restrict__ v_cache,
                                                            const int* __restrict__ block_tables, int bt_stride,
                                                            const int* __restrict__ seq_lens, int Hq, int G, int dk,
-                                                           int dv, int bs, float scale, int window, int sink) {
+                                                           int dv, int bs, float scale, int window, int sink,
+                                                           const float* __restrict__ sinks) {
   __shared__ float q_s[kMaxDK];
   __shared__ float p_s[64];
   const int b = blockIdx.x, h = blockIdx.y;
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
   }
   const int lo = window > 0 ? max(0, n - window) : 0;
   attend_wave<T>(o, qkv + (long)b * q_stride + (long)h * dk, k_cache, v_cache, block_tables + (long)b * bt_stride, lo,
-                 n, h / (Hq / G), G, dk, dv, bs, scale, sink, q_s, p_s);
+                 n, h / (Hq / G), G, dk, dv, bs, scale, sink, sinks != nullptr ? sinks[h] : 0.f, q_s, p_s);
 }
 
 // bf16 decode with 16-byte loads, 16-token pages: one workgroup (NW = 8 waves; 4 for 8 query heads
@@ -150,7 +152,8 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
                                                                 const bf16_t* __restrict__ v_cache,
                                                                 const int* __restrict__ block_tables, int bt_stride,
                                                                 const int* __restrict__ seq_lens, int Hq, int G, int dk,
-                                                                int dv, float scale, int window, int sink) {
+                                                                int dv, float scale, int window, int sink,
+                                                                const float* __restrict__ sinks) {
   constexpr int bs = 16;
   __shared__ __attribute__((aligned(16))) float q_s[R * kMaxDK];
   __shared__ __attribute__((aligned(16))) float p_s[NW][R][64];
@@ -172,7 +175,8 @@ __global__ __launch_bounds__(64 * NW) void window_decode_vec_kernel(bf16_t* __re
   float m[R], l[R], acc[R][kMaxVC];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    m[r] = first ? 0.f : -INFINITY;
+    // the sink's logit is not scaled; scores live in the base-2 domain
+    m[r] = first ? (sinks != nullptr ? sinks[g * R + r] * 1.44269504088896341f : 0.f) : -INFINITY;
     l[r] = first ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < kMaxVC; ++c) acc[r][c] = 0.f;
@@ -302,7 +306,7 @@ __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ qkv, long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
     const int* __restrict__ block_tables, int bt_stride, int S, int Hq, int G, float scale, int window,
-    int sink) {
+    int sink, const float* __restrict__ sinks) {
   // pages hold 16 tokens; scores live in the base-2 domain (scale * log2 e folded in) so that every
   // exponential is one v_exp_f32
   const float sc2 = scale * 1.44269504088896341f;
@@ -336,7 +340,7 @@ __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
     for (int ks = 0; ks < DK / 32; ++ks) qf[t][ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks + 8 * quad);
 #pragma unroll
     for (int dt = 0; dt < DV / 16; ++dt) oacc[t][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    m[t] = sink ? 0.f : -INFINITY;
+    m[t] = sink ? (sinks != nullptr ? sinks[blockIdx.y] * 1.44269504088896341f : 0.f) : -INFINITY;
     l[t] = sink ? 1.f : 0.f;
   }
   const int lo_t = window > 0 ? max(0, p0 - window + 1) : 0, hi = p0 + nq;
@@ -451,8 +455,8 @@ int k8sllm_hy_qk_norm_cache(void* qkv, long stride, const float* qw, const float
 
 int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                              const int* cu, const int* ctx, const int* block_tables, int bt_stride, int S, long T,
-                             int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink, int f32,
-                             int mfma, hipStream_t s) {
+                             int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink,
+                             const float* sinks, int f32, int mfma, hipStream_t s) {
   if (T <= 0 || S <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
   // bf16 with matrix-core head sizes and 16-byte aligned rows: the MFMA kernel
@@ -464,7 +468,7 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
 #define K8SLLM_WP(DK, DV, QT)                                                                                          \
   hipLaunchKernelGGL((window_prefill_mfma_kernel<DK, DV, QT>), grid, dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,  \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, block_tables, bt_stride, S, Hq, \
-                     G, scale, window, sink)
+                     G, scale, window, sink, sinks)
 #define K8SLLM_WPQ(DK, DV)                                       \
   if (qrows == 64) K8SLLM_WP(DK, DV, 4);                         \
   else if (qrows == 32) K8SLLM_WP(DK, DV, 2);                    \
@@ -481,17 +485,18 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
   if (f32)
     hipLaunchKernelGGL(window_prefill_kernel<float>, dim3(T, Hq), dim3(64), 0, s, (float*)out, (const float*)qkv,
                        q_stride, (const float*)k_cache, (const float*)v_cache, cu, ctx, block_tables, bt_stride, S, Hq,
-                       G, dk, dv, bs, scale, window, sink);
+                       G, dk, dv, bs, scale, window, sink, sinks);
   else
     hipLaunchKernelGGL(window_prefill_kernel<bf16_t>, dim3(T, Hq), dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,
                        q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, block_tables, bt_stride, S,
-                       Hq, G, dk, dv, bs, scale, window, sink);
+                       Hq, G, dk, dv, bs, scale, window, sink, sinks);
   return (int)hipGetLastError();
 }
 
 int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const void* k_cache, const void* v_cache,
                             const int* block_tables, int bt_stride, const int* seq_lens, int B, int Hq, int G, int dk,
-                            int dv, int bs, float scale, int window, int sink, int f32, int vec, hipStream_t s) {
+                            int dv, int bs, float scale, int window, int sink, const float* sinks, int f32, int vec,
+                            hipStream_t s) {
   if (B <= 0) return 0;
   if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
   const int R = Hq / G;
@@ -500,7 +505,7 @@ int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const voi
   hipLaunchKernelGGL((window_decode_vec_kernel<RR, (RR == 8 ? 4 : 8)>), dim3(B, G), dim3(RR == 8 ? 256 : 512), 0, s,     \
                      (bf16_t*)out, (const bf16_t*)qkv,                                                                  \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_stride, seq_lens, Hq, G, \
-                     dk, dv, scale, window, sink)
+                     dk, dv, scale, window, sink, sinks)
     if (R == 1) K8SLLM_WD(1);
     else if (R == 2) K8SLLM_WD(2);
     else if (R == 4) K8SLLM_WD(4);
@@ -511,11 +516,11 @@ int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const voi
   if (f32)
     hipLaunchKernelGGL(window_decode_kernel<float>, dim3(B, Hq), dim3(64), 0, s, (float*)out, (const float*)qkv,
                        q_stride, (const float*)k_cache, (const float*)v_cache, block_tables, bt_stride, seq_lens, Hq, G,
-                       dk, dv, bs, scale, window, sink);
+                       dk, dv, bs, scale, window, sink, sinks);
   else
     hipLaunchKernelGGL(window_decode_kernel<bf16_t>, dim3(B, Hq), dim3(64), 0, s, (bf16_t*)out, (const bf16_t*)qkv,
                        q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, bt_stride, seq_lens, Hq,
-                       G, dk, dv, bs, scale, window, sink);
+                       G, dk, dv, bs, scale, window, sink, sinks);
   return (int)hipGetLastError();
 }
 }

@@ -102,13 +102,15 @@ def add_norm(residual: torch.Tensor, addends: tuple, vec: Optional[torch.Tensor]
 
 def norm_shift(residual: torch.Tensor, addends: tuple, w: torch.Tensor, eps: float, one_plus: bool,
                mu: torch.Tensor, state: torch.Tensor, seg_cu: torch.Tensor, seg_ctx: torch.Tensor,
-               seg_slot: torch.Tensor, out_dtype: torch.dtype, advance: bool = True) -> torch.Tensor:
+               seg_slot: torch.Tensor, out_dtype: torch.dtype, advance: bool = True,
+               multi: bool = True) -> torch.Tensor:
     """Token-shifted norm.  ``residual`` (fp32 [T, d], updated in place) += ``addends``; with
     ``h[t]`` the RMSNorm of row t times ``w`` (fp32), returns ``h[t] + (h[t-1] - h[t]) * mu`` in
     ``out_dtype``, where the row before a segment's first comes from ``state[slot]`` ([slots, d]
     fp32; zeros where seg_ctx is 0).  ``advance``: ``state[slot]`` then takes the segment's last
     ``h`` (unshifted).  GPU: the state of segments longer than one row is advanced by a second
-    small launch, after every row has read the old state."""
+    small launch, after every row has read the old state (``multi`` False: the caller knows every
+    segment is one row, as in a decode step, and that launch is left out)."""
     if not residual.is_cuda:
         for a in addends:
             residual += a.float()
@@ -126,11 +128,11 @@ def norm_shift(residual: torch.Tensor, addends: tuple, w: torch.Tensor, eps: flo
             if advance and slot >= 0:
                 state[slot] = h[b - 1]
         return (h + (prev - h) * mu.float()).to(out_dtype)
-    assert len(addends) <= 2
+    for a in addends:  # a row also norms its predecessor, so the stream is complete before the launch
+        residual += a
     out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
-    a = list(addends) + [None] * (2 - len(addends))
-    native().norm_shift(out, residual, a[0], a[1], w, float(eps), bool(one_plus), mu, state, seg_cu, seg_ctx, seg_slot,
-                        bool(advance))
+    native().norm_shift(out, residual, w, float(eps), bool(one_plus), mu, state, seg_cu, seg_ctx, seg_slot,
+                        bool(advance), bool(multi))
     return out
 
 
@@ -275,26 +277,30 @@ def window_attention_decode(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: t
 
 # ---------------------------------------------------------------- latent attention
 
-def _rotate_half(v: torch.Tensor, pos: torch.Tensor, base: float, dims: int) -> torch.Tensor:
-    """v [T, ..., n] fp32: the first ``dims`` entries of the last axis turn in pairs (i, i + dims/2) by
-    the angle pos * base^(-2i/dims) (angles in fp32); the rest pass."""
-    half = dims // 2
-    f = torch.pow(torch.tensor(float(base), dtype=torch.float64),
-                  -2.0 * torch.arange(half, dtype=torch.float64) / dims).float().to(v.device)
-    a = pos.float().view(-1, *([1] * (v.dim() - 1))) * f
+def rotary_freq(base: float, dims: int, device=None) -> torch.Tensor:
+    """The ``dims / 2`` rotation frequencies base^(-2i/dims) as fp32 (evaluated in float64)."""
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * torch.arange(dims // 2, dtype=torch.float64) / dims)
+    return f.float().to(device) if device is not None else f.float()
+
+
+def _rotate_half(v: torch.Tensor, pos: torch.Tensor, freq: torch.Tensor) -> torch.Tensor:
+    """v [T, ..., n] fp32: with nf = len(freq), entries i and i + nf of the last axis (i < nf) turn by
+    the angle pos * freq[i] (angles in fp32); entries from 2 nf on pass."""
+    half = freq.numel()
+    a = pos.float().view(-1, *([1] * (v.dim() - 1))) * freq.float()
     c, s = torch.cos(a), torch.sin(a)
-    u, x = v[..., :half], v[..., half:dims]
-    return torch.cat([u * c - x * s, x * c + u * s, v[..., dims:]], -1)
+    u, x = v[..., :half], v[..., half:2 * half]
+    return torch.cat([u * c - x * s, x * c + u * s, v[..., 2 * half:]], -1)
 
 
 def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw: torch.Tensor,
-                kw: Optional[torch.Tensor], eps: float, positions: torch.Tensor, base: float, dims: int,
+                kw: Optional[torch.Tensor], eps: float, positions: torch.Tensor, freq: torch.Tensor,
                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                 slot_mapping: Optional[torch.Tensor]) -> None:
     """In place on the fused down-projections [T, q_rank | kv_rank | rot_dim] (or [T, q_rank] for a
     layer that reads another layer's cache): the query latent is RMS-normed (weight ``qw``); the
     key/value latent is RMS-normed (weight ``kw``) and the shared key part behind it is rotated by
-    its position; both go to the pages at ``slot_mapping`` - the key page row is [latent | rotated
+    its position (``freq``: rotary_freq); both go to the pages at ``slot_mapping`` - the key page row is [latent | rotated
     part], the value page holds the latent once more, dim-major."""
     T = proj.shape[0]
     if not proj.is_cuda:
@@ -304,7 +310,7 @@ def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw:
             return
         c = proj[:, q_rank:q_rank + kv_rank].float()
         c = (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kw.float()).to(proj.dtype)
-        kr = _rotate_half(proj[:, q_rank + kv_rank:].float(), positions, base, dims).to(proj.dtype)
+        kr = _rotate_half(proj[:, q_rank + kv_rank:].float(), positions, freq).to(proj.dtype)
         proj[:, q_rank:q_rank + kv_rank] = c
         proj[:, q_rank + kv_rank:] = kr
         ok = slot_mapping >= 0
@@ -313,22 +319,22 @@ def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw:
         k_cache.view(-1, kv_rank + rot_dim)[s] = proj[ok, q_rank:]
         v_cache.view(-1, kv_rank, bs)[s // bs, :, s % bs] = c[ok]
         return
-    native().latent_prep(proj, int(q_rank), int(kv_rank), int(rot_dim), qw, kw, float(eps), positions, float(base),
-                         int(dims), k_cache, v_cache, slot_mapping)
+    native().latent_prep(proj, int(q_rank), int(kv_rank), int(rot_dim), qw, kw, float(eps), positions, freq,
+                         k_cache, v_cache, slot_mapping)
 
 
 def latent_queries(q: torch.Tensor, q_lat: torch.Tensor, H: int, dim: int, rot_dim: int, positions: torch.Tensor,
-                   base: float, dims: int) -> torch.Tensor:
+                   freq: torch.Tensor) -> torch.Tensor:
     """The queries against the latent cache: per head [q_lat | rotated part], [T, H * (R + rot_dim)].
     ``q`` [T, H * (dim + rot_dim)] are the up-projected queries (their last ``rot_dim`` entries per
     head are rotated by the position) and ``q_lat`` [H, T, R] the unrotated parts already
     multiplied into the latent space."""
     T, R = q.shape[0], q_lat.shape[2]
     if not q.is_cuda:
-        qr = _rotate_half(q.view(T, H, dim + rot_dim)[..., dim:].float(), positions, base, dims).to(q.dtype)
+        qr = _rotate_half(q.view(T, H, dim + rot_dim)[..., dim:].float(), positions, freq).to(q.dtype)
         return torch.cat([q_lat.transpose(0, 1), qr], -1).reshape(T, H * (R + rot_dim))
     out = torch.empty(T, H * (R + rot_dim), dtype=q.dtype, device=q.device)
-    native().latent_queries(out, q, q_lat, int(H), int(dim), int(rot_dim), positions, float(base), int(dims))
+    native().latent_queries(out, q, q_lat, int(H), int(dim), int(rot_dim), positions, freq)
     return out
 
 
