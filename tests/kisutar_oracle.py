@@ -192,3 +192,13 @@ def random_weights(cfg: dict, seed: int = 0) -> dict:
                 fs = ml["shared"]["ff"]
                 w[P + "shared.up"], w[P + "shared.down"] = rnd(fs, d, std=d ** -0.5), rnd(d, fs, std=fs ** -0.5)
     return w
+
+
+def greedy(cfg: dict, w: dict, prompt, n: int) -> list:
+    """``n`` tokens by repeated whole-sequence forwards, each the argmax of the last logits."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = int(torch.argmax(forward(cfg, w, seq)[-1]))
+        out.append(t)
+        seq.append(t)
+    return out

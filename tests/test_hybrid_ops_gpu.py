@@ -254,3 +254,144 @@ def test_experts_matrix_core_paths(T, E, K, d, ff, il):
     for mfma in (True, False):
         got = H.moe_experts(h.cuda(), ids.cuda(), w.cuda(), w13g.cuda(), w2.cuda(), sh.cuda(), gate.cuda(), il=il, mfma=mfma)
         torch.testing.assert_close(got.cpu(), want, **_tol(dt))
+
+
+# ---------------------------------------------------------------- sequential-block designs' operators
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("d", [72, 70, 2304])
+def test_norm_shift_and_state(dt, d):
+    """Segments of several rows and of one row, continuing from a slot or fresh, a padding segment;
+    the state after the step; both steps of a prompt cut in two give the rows of the whole."""
+    g = _g(11)
+    T = 12
+    x, w, mu = _r(g, T, d), _r(g, d, s=0.2) + 1, torch.rand(d, generator=g)
+    cu, ctx, slot = _i32([0, 5, 6, 7, 12]), _i32([0, 9, 0, 3]), _i32([2, 0, -1, 1])
+    st = _r(g, 4, d)
+    for one_plus in (False, True):
+        s_c, s_g = st.clone(), st.clone().cuda()
+        want = H.norm_shift(x.clone(), (), w, 1e-6, one_plus, mu, s_c, cu, ctx, slot, dt)
+        got = H.norm_shift(x.clone().cuda(), (), w.cuda(), 1e-6, one_plus, mu.cuda(), s_g, cu.cuda(), ctx.cuda(), slot.cuda(), dt)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+        torch.testing.assert_close(s_g.cpu(), s_c, rtol=1e-5, atol=1e-5)
+        assert torch.equal(s_g.cpu()[3], st[3])
+    a = _r(g, T, d, dt=dt)
+    s_c, s_g = st.clone(), st.clone().cuda()
+    r_c, r_g = x.clone(), x.clone().cuda()
+    want = H.norm_shift(r_c, (a,), w, 1e-6, False, mu, s_c, cu, ctx, slot, dt)
+    got = H.norm_shift(r_g, (a.cuda(),), w.cuda(), 1e-6, False, mu.cuda(), s_g, cu.cuda(), ctx.cuda(), slot.cuda(), dt)
+    torch.testing.assert_close(r_g.cpu(), r_c, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+    # one-row segments only (a decode step): no second launch
+    cu1, ctx1, slot1 = torch.arange(T + 1, dtype=torch.int32), _i32([0, 3] * 6), _i32([2, 0, -1, 3, -1, 1] + [-1] * 6)
+    s_c, s_g = st.clone(), st.clone().cuda()
+    want = H.norm_shift(x.clone(), (), w, 1e-6, False, mu, s_c, cu1, ctx1, slot1, dt)
+    got = H.norm_shift(x.clone().cuda(), (), w.cuda(), 1e-6, False, mu.cuda(), s_g, cu1.cuda(), ctx1.cuda(), slot1.cuda(), dt,
+                       multi=False)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("n", [0, 1, 7])
+def test_depth_mix(n):
+    g = _g(12)
+    T, d = 9, 36
+    for add_dt in (None, torch.float32, torch.bfloat16):
+        stack = _r(g, n + 3, T, d)
+        coef = _r(g, n + 1)
+        add = _r(g, T, d, dt=add_dt) if add_dt is not None else None
+        s_c, s_g = stack.clone(), stack.clone().cuda()
+        want = H.depth_mix(s_c, n, add, coef)
+        got = H.depth_mix(s_g, n, add.cuda() if add is not None else None, coef.cuda())
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(s_g.cpu(), s_c, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("kind", ["gelu", "gelu_tanh", "xielu"])
+def test_activation(dt, kind):
+    g = _g(13)
+    for shape in ((5, 37), (3, 64)):
+        x = _r(g, *shape, s=3.0, dt=dt)
+        want = H.activation(x, kind, 0.6, 0.9)
+        got = H.activation(x.cuda(), kind, 0.6, 0.9)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("Q,R,dr,nf", [(20, 24, 8, 4), (300, 520, 6, 2), (8, 8, 2, 1)])
+def test_latent_prep_and_queries(dt, Q, R, dr, nf):
+    g = _g(14)
+    T, H_, dn, bs, nb = 11, 3, 10, 16, 6
+    proj = _r(g, T, Q + R + dr, dt=dt)
+    qw, kw = _r(g, Q, s=0.2) + 1, _r(g, R, s=0.2) + 1
+    pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
+    freq = H.rotary_freq(1000.0, 2 * nf)
+    slots = _i32([17, 3, -1, 95, 64, 0, 33, 34, 35, 80, 15])
+    kc, vc = torch.zeros(nb, bs, R + dr, dtype=dt), torch.zeros(nb, 1, R, bs, dtype=dt)
+    p_c, p_g, kg, vg = proj.clone(), proj.clone().cuda(), kc.clone().cuda(), vc.clone().cuda()
+    H.latent_prep(p_c, Q, R, dr, qw, kw, 1e-6, pos, freq, kc, vc, slots)
+    H.latent_prep(p_g, Q, R, dr, qw.cuda(), kw.cuda(), 1e-6, pos.cuda(), freq.cuda(), kg, vg, slots.cuda())
+    tol = _tol(dt)
+    torch.testing.assert_close(p_g.cpu().float(), p_c.float(), **tol)
+    torch.testing.assert_close(kg.cpu().float(), kc.float(), **tol)
+    torch.testing.assert_close(vg.cpu().float(), vc.float(), **tol)
+    # a layer without key/value projection: only the query latent is normed
+    p2 = proj[:, :Q].contiguous()
+    p2c, p2g = p2.clone(), p2.clone().cuda()
+    H.latent_prep(p2c, Q, R, dr, qw, None, 1e-6, pos, freq, None, None, None)
+    H.latent_prep(p2g, Q, R, dr, qw.cuda(), None, 1e-6, pos.cuda(), freq.cuda(), None, None, None)
+    torch.testing.assert_close(p2g.cpu().float(), p2c.float(), **tol)
+    q, ql = _r(g, T, H_ * (dn + dr), dt=dt), _r(g, H_, T, R, dt=dt)
+    want = H.latent_queries(q, ql, H_, dn, dr, pos, freq)
+    got = H.latent_queries(q.cuda(), ql.cuda(), H_, dn, dr, pos.cuda(), freq.cuda())
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_attention_with_learned_sinks(dt):
+    """Per-head sink logits in all four attention kernels (any-size and matrix-core prefill, any-size
+    and vector decode) against the torch form."""
+    g = _g(15)
+    for Hq, G, dk, dv in ((8, 1, 104, 80), (4, 2, 64, 64), (3, 1, 20, 12)):
+        lens, chunk = [50, 9, 33], [20, 9, 2]
+        kc, vc, bt = _paged(g, dt, lens, Hq, G, dk, dv)
+        sinks = _r(g, Hq, s=2.0)
+        T = sum(chunk)
+        qkv = _r(g, T, Hq * dk, s=0.3, dt=dt)
+        cu = _i32([0, 20, 29, 31])
+        ctx = _i32([n - c for n, c in zip(lens, chunk)])
+        a = (Hq, G, dk, dv, 0.2, 24, True)
+        want = H.window_attention_prefill(qkv, kc, vc, cu, ctx, bt, *a, sinks=sinks)
+        base = H.window_attention_prefill(qkv, kc, vc, cu, ctx, bt, *a)
+        assert float((want.float() - base.float()).abs().max()) > 1e-2  # the sinks are not a no-op
+        dev = [t.cuda() for t in (qkv, kc, vc, cu, ctx, bt)]
+        for mode in (1, 0):
+            got = H.window_attention_prefill(*dev, *a, mfma=mode, sinks=sinks.cuda())
+            torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+        q1 = _r(g, 3, Hq * dk, s=0.3, dt=dt)
+        sl = _i32(lens)
+        want = H.window_attention_decode(q1, kc, vc, bt, sl, *a, sinks=sinks)
+        for vec in (True, False):
+            got = H.window_attention_decode(q1.cuda(), kc.cuda(), vc.cuda(), bt.cuda(), sl.cuda(), *a, vec=vec, sinks=sinks.cuda())
+            torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_router_over_all_and_gelu_experts(dt):
+    g = _g(16)
+    T, d, E, K, ff = 37, 64, 6, 3, 48
+    h = _r(g, T, d, dt=dt)
+    wr = _r(g, E, d, s=0.3)
+    ids_c, w_c, _ = H.moe_router(h, wr, None, E, K, over_all=True)
+    ids_g, w_g, gate = H.moe_router(h.cuda(), wr.cuda(), None, E, K, over_all=True)
+    assert gate is None and torch.equal(ids_g.cpu(), ids_c)
+    torch.testing.assert_close(w_g.cpu(), w_c, rtol=1e-5, atol=1e-6)
+    assert float(w_c.sum(-1).max()) < 1.0
+    w1, w2 = _r(g, E, ff, d, s=d ** -0.5, dt=dt), _r(g, E, d, ff, s=ff ** -0.5, dt=dt)
+    shared = _r(g, T, d, dt=dt)
+    for sh in (None, shared):
+        want = H.moe_experts(h, ids_c, w_c, w1, w2, sh, None, act="gelu")
+        for mfma in (True, False):
+            got = H.moe_experts(h.cuda(), ids_g, w_g, w1.cuda(), w2.cuda(), sh.cuda() if sh is not None else None, None,
+                                act="gelu", mfma=mfma)
+            torch.testing.assert_close(got.cpu(), want, **_tol(dt))
