@@ -192,6 +192,7 @@ class LatentAttention:
         self.kv_from = None if self.kv_from is None else int(self.kv_from)
         self.eps = eps
         self.fast = 1
+        self.pitch = (self.R + self.dr + 31) // 32 * 32
         H, dn, dr, dv, Q, R = self.H, self.dn, self.dr, self.dv, self.Q, self.R
         wd = [p.get(prefix + "dq", (Q, d), 1.0 / math.sqrt(d))]
         self.kn = None
@@ -210,11 +211,12 @@ class LatentAttention:
     def new_cache(self, num_blocks: int, num_slots: int, dtype, device) -> dict:
         if self.kv_from is not None:
             return {}
-        return {"k": torch.zeros(num_blocks, BLOCK, self.R + self.dr, dtype=dtype, device=device),
+        # key rows [latent | rotated part], padded with zeros to the matrix-core kernel's multiple of 32
+        return {"k": torch.zeros(num_blocks, BLOCK, self.pitch, dtype=dtype, device=device),
                 "v": torch.zeros(num_blocks, 1, self.R, BLOCK, dtype=dtype, device=device)}
 
     def cache_bytes(self, esize: int) -> tuple:
-        return (0 if self.kv_from is not None else BLOCK * (2 * self.R + self.dr) * esize), 0
+        return (0 if self.kv_from is not None else BLOCK * (self.pitch + self.R) * esize), 0
 
     def forward(self, h: torch.Tensor, meta: AttnMeta, cache: dict) -> torch.Tensor:
         H, dn, dr, dv, Q, R = self.H, self.dn, self.dr, self.dv, self.Q, self.R
@@ -227,18 +229,17 @@ class LatentAttention:
         q = F.linear(down[:, :Q], self.w_uq)
         # the per-head key expansion moved to the query: q_lat[h] = q_unrotated[h] @ W_uk[h]  ([H, T, R])
         q_lat = torch.bmm(q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1), self.w_uk.view(H, dn, R))
-        qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.freq)
-        args = (H, 1, R + dr, R, self.scale, self.window, True)
+        qa = hops.latent_queries(q, q_lat, H, dn, dr, meta.positions, self.freq, self.pitch)
+        args = (H, self.scale, self.window, self.sinks)
         if not meta.is_prefill:
-            o = hops.window_attention_decode(qa, kc, vc, meta.block_tables, meta.seq_lens, *args, vec=bool(self.fast),
-                                             sinks=self.sinks)
+            o = hops.latent_attention(qa, kc, vc, meta.block_tables, *args, seq_lens=meta.seq_lens, fast=self.fast)
         else:
             nd = meta.num_decode
-            o = hops.window_attention_prefill(qa[nd:], kc, vc, meta.cu_seqlens, meta.ctx_start, meta.block_tables,
-                                              *args, mfma=self.fast, sinks=self.sinks)
+            o = hops.latent_attention(qa[nd:], kc, vc, meta.block_tables, *args, cu=meta.cu_seqlens, ctx=meta.ctx_start,
+                                      fast=self.fast)
             if nd:
-                od = hops.window_attention_decode(qa[:nd], kc, vc, meta.dec_block_tables, meta.dec_seq_lens, *args,
-                                                  vec=bool(self.fast), sinks=self.sinks)
+                od = hops.latent_attention(qa[:nd], kc, vc, meta.dec_block_tables, *args, seq_lens=meta.dec_seq_lens,
+                                           fast=self.fast)
                 o = torch.cat([od, o])
         # ... and the value expansion to the result: v[h] = o_lat[h] @ W_uv[h]^T, written head by head
         # into the rows the out-projection reads

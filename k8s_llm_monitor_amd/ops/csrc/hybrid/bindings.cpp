@@ -44,10 +44,14 @@ int k8sllm_hy_depth_mix(float* stack, long plane, int n, const void* addend, int
                         hipStream_t s);
 int k8sllm_hy_activation(void* out, const void* x, long n, int kind, float a, float b, int f32, hipStream_t s);
 int k8sllm_hy_latent_prep(void* proj, long stride, long T, int Q, int R, int dr, const float* qw, const float* kw,
-                          float eps, const int* positions, const float* freq, int nf, void* k_cache, void* v_cache,
-                          const int* slots, int bs, int f32, hipStream_t s);
+                          float eps, const int* positions, const float* freq, int nf, void* k_cache, int kw_pitch,
+                          void* v_cache, const int* slots, int bs, int f32, hipStream_t s);
 int k8sllm_hy_latent_queries(void* out, const void* q, long q_stride, const void* q_lat, long T, int H, int dn, int dr,
-                             int R, const int* positions, const float* freq, int nf, int f32, hipStream_t s);
+                             int R, int w, const int* positions, const float* freq, int nf, int f32, hipStream_t s);
+int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const void* k_cache, const void* v_cache,
+                               const int* cu, const int* ctx, const int* seq_lens, const int* block_tables,
+                               int bt_stride, int S, long T, int H, int dkp, int dv, int bs, float scale, int window,
+                               const float* sinks, int split, hipStream_t s);
 int k8sllm_moe_align(const int* topk_ids, long n, int E, int* expert_offsets, int* sorted_idx, int* inv_idx,
                      hipStream_t s);
 }
@@ -443,14 +447,16 @@ void latent_prep(Tensor proj, int64_t Q, int64_t R, int64_t dr, Tensor qw, OptT 
   void *kc = nullptr, *vc = nullptr;
   const int* sp = nullptr;
   const float* kwp = nullptr;
-  int bs = 16;
+  int bs = 16, pitch = 0;
   if (own) {
     f32c(*kw, "dkv.norm");
     TORCH_CHECK(kw->numel() == R, "dkv.norm [kv_rank]");
     kwp = kw->data_ptr<float>();
     if (k_cache.has_value()) {
       TORCH_CHECK(v_cache.has_value() && slots.has_value(), "k_cache, v_cache and slot_mapping come together");
-      pages(*k_cache, f, R + dr, "k_cache");
+      TORCH_CHECK(k_cache->dim() == 3 && k_cache->size(2) >= R + dr, "k_cache rows hold [latent | rotated part]");
+      pitch = (int)k_cache->size(2);
+      pages(*k_cache, f, pitch, "k_cache");
       vpages(*v_cache, *k_cache, f, 1, R);
       sp = iptr(slots, "slot_mapping");
       TORCH_CHECK(slots->numel() >= T, "slot_mapping [T]");
@@ -460,8 +466,8 @@ void latent_prep(Tensor proj, int64_t Q, int64_t R, int64_t dr, Tensor qw, OptT 
     }
   }
   check(k8sllm_hy_latent_prep(proj.data_ptr(), proj.stride(0), T, (int)Q, (int)R, (int)dr, qw.data_ptr<float>(), kwp,
-                              (float)eps, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), kc, vc, sp,
-                              bs, f, cur()),
+                              (float)eps, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), kc, pitch, vc,
+                              sp, bs, f, cur()),
         "latent_prep");
 }
 
@@ -475,11 +481,50 @@ void latent_queries(Tensor out, Tensor q, Tensor q_lat, int64_t H, int64_t dn, i
   TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * (dn + dr), "q [T, H * (dim + rot)]");
   TORCH_CHECK(q_lat.dim() == 3 && q_lat.is_contiguous() && q_lat.size(0) == H && q_lat.size(1) == T, "q_lat [H, T, R]");
   const int64_t R = q_lat.size(2);
-  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * (R + dr) && positions.numel() >= T && 2 * freq.numel() <= dr,
-              "latent_queries: out / positions / freq");
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && out.size(0) == T && out.size(1) % H == 0 && out.size(1) / H >= R + dr &&
+                  positions.numel() >= T && 2 * freq.numel() <= dr,
+              "latent_queries: out [T, H * pitch] / positions / freq");
   check(k8sllm_hy_latent_queries(out.data_ptr(), q.data_ptr(), q.stride(0), q_lat.data_ptr(), T, (int)H, (int)dn, (int)dr,
-                                 (int)R, positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(), f, cur()),
+                                 (int)R, (int)(out.size(1) / H), positions.data_ptr<int>(), freq.data_ptr<float>(), (int)freq.numel(),
+                                 f, cur()),
         "latent_queries");
+}
+
+// The matrix-core latent attention; false: these sizes or dtype are not the kernel's, nothing was
+// launched.  cu / ctx given: prompt chunks (block_tables per segment); else one row per sequence.
+bool latent_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, OptT cu, OptT ctx, OptT seq_lens,
+                      Tensor block_tables, int64_t H, double scale, int64_t window, OptT sinks, int64_t split) {
+  if (act(q, "q") != 0) return false;
+  same(out, 0, "out");
+  TORCH_CHECK(k_cache.dim() == 3 && v_cache.dim() == 4, "pages");
+  const int64_t dkp = k_cache.size(2), dv = v_cache.size(2), T = q.size(0);
+  pages(k_cache, 0, dkp, "k_cache");
+  vpages(v_cache, k_cache, 0, 1, dv);
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) == H * dkp, "q [T, H * key pitch]");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * dv, "out [T, H * dv]");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == torch::kInt32 && block_tables.dim() == 2 &&
+                  block_tables.stride(1) == 1,
+              "block_tables [S, W] int32");
+  const int *cup = nullptr, *ctxp = nullptr, *slp = nullptr;
+  int64_t S = 0;
+  if (cu.has_value()) {
+    TORCH_CHECK(ctx.has_value(), "cu and ctx come together");
+    cup = iptr(cu, "cu");
+    ctxp = iptr(ctx, "ctx");
+    S = ctx->numel();
+    TORCH_CHECK(cu->numel() == S + 1 && block_tables.size(0) >= S, "cu [S+1], block_tables [S, W]");
+  } else {
+    slp = iptr(seq_lens, "seq_lens");
+    TORCH_CHECK(slp != nullptr && seq_lens->numel() >= T && block_tables.size(0) >= T, "seq_lens [T], block_tables [T, W]");
+  }
+  TORCH_CHECK(window >= 0 && H >= 1, "heads / window");
+  const int rc = k8sllm_hy_latent_attention(out.data_ptr(), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+                                            cup, ctxp, slp, block_tables.data_ptr<int>(), (int)block_tables.stride(0), (int)S, T,
+                                            (int)H, (int)dkp, (int)dv, (int)k_cache.size(1), (float)scale, (int)window,
+                                            sink_ptr(sinks, H), (int)split, cur());
+  if (rc == 1) return false;
+  check(rc, "latent_attention");
+  return true;
 }
 
 }  // namespace
@@ -503,4 +548,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("activation", &activation);
   m.def("latent_prep", &latent_prep);
   m.def("latent_queries", &latent_queries);
+  m.def("latent_attention", &latent_attention);
 }

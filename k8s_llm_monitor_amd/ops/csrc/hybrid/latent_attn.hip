@@ -1,9 +1,11 @@
 // Latent (low-rank compressed) attention: what surrounds the attention kernels of window_attn.hip.
 //   latent_prep     in place on the fused down-projections [T][q_rank | kv_rank | rot]: RMSNorm of the
 //                   query latent; RMSNorm of the key/value latent and rotation of the shared key part,
-//                   both written to the pages: key page row = [latent | rotated part], value page =
-//                   the latent once more, dim-major ([blocks][1][kv_rank][BS])
-//   latent_queries  per head [q_lat (unrotated query times the key expansion) | rotated query part]
+//                   both written to the pages: key page row = [latent | rotated part | zeros up to the
+//                   row pitch], value page = the latent once more, dim-major ([blocks][1][kv_rank][BS])
+//   latent_queries  per head [q_lat (unrotated query times the key expansion) | rotated query part |
+//                   zeros up to the same pitch]
+//   latent_attention  the matrix-core attention over those pages (bf16), prompt chunks and decoding
 // Rotation: entries i and i + n/2 of the first 2 * nf entries (nf frequencies, freq[i] given in fp32)
 // turn by the angle position * freq[i]; angles, sine and cosine are fp32.
 #include "hy_common.h"
@@ -15,7 +17,8 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ proj, 
                                                           const float* __restrict__ qw, const float* __restrict__ kw,
                                                           float eps, const int* __restrict__ positions,
                                                           const float* __restrict__ freq, int nf,
-                                                          T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                          T* __restrict__ k_cache, int kw_pitch,
+                                                          T* __restrict__ v_cache,
                                                           const int* __restrict__ slots, int bs) {
   __shared__ float red[4];
   const long t = blockIdx.x;
@@ -36,7 +39,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ proj, 
   sc = block_sum<256>(sc, red);
   const float ic = 1.0f / sqrtf(sc / (float)R + eps);
   const long slot = (slots != nullptr && k_cache != nullptr) ? slots[t] : -1;
-  T* kp = slot >= 0 ? k_cache + slot * (long)(R + dr) : nullptr;
+  T* kp = slot >= 0 ? k_cache + slot * (long)kw_pitch : nullptr;  // the pitch's tail stays zero
   for (int c = threadIdx.x; c < R; c += 256) {
     T* e = row + Q + c;
     stf(e, ldf(e) * ic * kw[c]);
@@ -67,14 +70,17 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ proj, 
 template <typename T>
 __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out, const T* __restrict__ q, long q_stride,
                                                              const T* __restrict__ q_lat, long T_rows, int H, int dn,
-                                                             int dr, int R, const int* __restrict__ positions,
+                                                             int dr, int R, int w, const int* __restrict__ positions,
                                                              const float* __restrict__ freq, int nf) {
   const long t = blockIdx.x;
-  const int w = R + dr;
   const float pos = (float)positions[t];
   T* o = out + t * (long)H * w;
-  for (int c = threadIdx.x; c < H * w; c += 256) {
+  for (int c = threadIdx.x; c < H * w; c += 256) {  // w >= R + dr: the row's pitch, zeros behind the query
     const int h = c / w, j = c - h * w;
+    if (j >= R + dr) {
+      stf(o + c, 0.f);
+      continue;
+    }
     if (j < R) {
       o[c] = q_lat[((long)h * T_rows + t) * R + j];
       continue;
@@ -93,6 +99,176 @@ __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out
   }
 }
 
+
+// bf16 latent attention on the matrix cores, prompt chunks and decoding alike.  All heads read the
+// same key/value stream, so the 16 query columns of a tile are 16 HEADS of ONE token (the window
+// mask is then the same for the whole tile), and a workgroup is (token, group of 16 heads):
+//   S^T[key][head] = K Q^T     v_mfma_f32_16x16x32_bf16: A = key rows, 16-byte loads from the page
+//                              ([latent | rotated part], padded with zeros to a multiple of 32),
+//                              B = the token's query rows, in registers for the whole loop
+//   O^T[d][head]  += V^T P^T   v_mfma_f32_16x16x16_bf16: B = the score accumulator itself, A = V^T,
+//                              8-byte loads from the dim-major latent page
+// The NW waves of a workgroup take the window's 16-key tiles in turn (decoding: the window is the
+// only parallel axis of a row) and merge their (maximum, denominator, output) through LDS: the common
+// maximum first, then the outputs summed wave after wave into one buffer.  Only wave 0 starts from
+// the sink.  Scores, weights and sums are fp32, base-2 exponentials (the scale carries log2 e).
+// KS_MAX / DT_MAX bound the key width / 32 and the value width / 16 (register arrays); the real
+// widths are run-time (wave-uniform guards).  cu == nullptr: one row per sequence at seq_lens - 1.
+template <int KS_MAX, int DT_MAX, int NW>
+__global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
+    const int* __restrict__ seq_lens, const int* __restrict__ block_tables, int bt_stride, int S, int H, int dkp,
+    int dv, float scale, int window, const float* __restrict__ sinks) {
+  constexpr int OP = DT_MAX * 16 + 4;  // LDS row pitch of the merge buffer (floats)
+  __shared__ __attribute__((aligned(16))) float o_s[NW > 1 ? 16 * OP : 4];
+  __shared__ float m_s[NW > 1 ? NW : 1][16];
+  __shared__ float l_s[NW > 1 ? NW : 1][16];
+  const float sc2 = scale * 1.44269504088896341f;
+  const int row = blockIdx.x, hg = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, quad = lane >> 4;
+  int s, p;
+  if (cu != nullptr) {
+    s = find_segment(cu, S, row);
+    p = ctx[s] + row - cu[s];
+  } else {
+    s = row;
+    p = seq_lens[row] - 1;
+  }
+  const int nh = min(16, H - hg * 16);
+  bf16_t* obase = out + ((long)row * H + hg * 16) * dv;
+  if (p < 0) {  // padding row of a decode bucket
+    for (int c = threadIdx.x; c < nh * dv; c += 64 * NW) obase[c] = 0;
+    return;
+  }
+  const int nks = dkp >> 5, ndt = dv >> 4;
+  const int head = hg * 16 + min(c16, nh - 1);
+  const int* bt = block_tables + (long)s * bt_stride;
+  const int lo = window > 0 ? max(0, p - window + 1) : 0, hi = p + 1;
+  bf16x8 qf[KS_MAX];
+  {
+    const bf16_t* qrow = q + (long)row * q_stride + (long)head * dkp + 8 * quad;
+#pragma unroll
+    for (int ks = 0; ks < KS_MAX; ++ks)
+      if (ks < nks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
+  }
+  f32x4 oacc[DT_MAX];
+#pragma unroll
+  for (int dt = 0; dt < DT_MAX; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  if (wave == 0) {
+    m = sinks != nullptr ? sinks[head] * 1.44269504088896341f : 0.f;
+    l = 1.f;
+  }
+  const bf16_t* kbase = k_cache + 8 * quad;
+  const bf16_t* vbase = v_cache + (long)c16 * 16 + 4 * quad;
+  const long vpage = (long)dv * 16;
+  const int jfirst = (lo & ~15) + 16 * wave;
+  bf16x8 kf_n[KS_MAX];
+  s16x4 vf_n[DT_MAX];
+  auto issue = [&](int j0) {
+    const long pg = bt[j0 >> 4];
+    const bf16_t* krow = kbase + ((pg << 4) + (min(j0 + c16, hi - 1) & 15)) * dkp;
+#pragma unroll
+    for (int ks = 0; ks < KS_MAX; ++ks)
+      if (ks < nks) kf_n[ks] = *reinterpret_cast<const bf16x8*>(krow + 32 * ks);
+    const bf16_t* vpg = vbase + pg * vpage;
+#pragma unroll
+    for (int dt = 0; dt < DT_MAX; ++dt)
+      if (dt < ndt) vf_n[dt] = *reinterpret_cast<const s16x4*>(vpg + dt * 256);
+  };
+  if (jfirst < hi) issue(jfirst);
+  for (int j0 = jfirst; j0 < hi; j0 += 16 * NW) {
+    bf16x8 kf[KS_MAX];
+    s16x4 vf[DT_MAX];
+#pragma unroll
+    for (int ks = 0; ks < KS_MAX; ++ks) kf[ks] = kf_n[ks];
+#pragma unroll
+    for (int dt = 0; dt < DT_MAX; ++dt) vf[dt] = vf_n[dt];
+    if (j0 + 16 * NW < hi) issue(j0 + 16 * NW);
+    f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS_MAX; ++ks)
+      if (ks < nks) sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], sacc, 0, 0, 0);
+    float sv[4], tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, head c16
+      const int j = j0 + 4 * quad + i;
+      sv[i] = (j >= lo && j < hi) ? sacc[i] * sc2 : -INFINITY;
+      tmax = fmaxf(tmax, sv[i]);
+    }
+    tmax = xor32_max_f(xor16_max(tmax));
+    const float mn = fmaxf(m, tmax);  // the tile holds at least one live key
+    const float alpha = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mn);
+    float ps = 0.f;
+    s16x4 pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float pv = sv[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sv[i] - mn);
+      ps += pv;
+      pb[i] = (short)f2bf(pv);
+    }
+    ps = xor32_sum_f(xor16_sum(ps));
+    l = l * alpha + ps;
+    m = mn;
+    const bool rescale = __any(alpha != 1.f);
+#pragma unroll
+    for (int dt = 0; dt < DT_MAX; ++dt)
+      if (dt < ndt) {
+        if (rescale) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
+        }
+        oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[dt], pb, oacc[dt], 0, 0, 0);
+      }
+  }
+  // oacc[dt][i] = O[head c16][d = 16 dt + 4 quad + i]
+  if (NW == 1) {
+    if (c16 >= nh) return;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* orow = obase + (long)c16 * dv;
+#pragma unroll
+    for (int dt = 0; dt < DT_MAX; ++dt)
+      if (dt < ndt) {
+        uint2 w;
+        w.x = pack2(oacc[dt][0] * inv, oacc[dt][1] * inv);
+        w.y = pack2(oacc[dt][2] * inv, oacc[dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * quad) = w;
+      }
+    return;
+  }
+  if (quad == 0) m_s[wave][c16] = m;
+  __syncthreads();
+  float M = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, m_s[w][c16]);  // wave 0's is finite (the sink)
+  const float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);
+  if (quad == 0) l_s[wave][c16] = l * f;
+  for (int w = 0; w < NW; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int dt = 0; dt < DT_MAX; ++dt)
+        if (dt < ndt) {
+          float4* dst = reinterpret_cast<float4*>(&o_s[c16 * OP + 16 * dt + 4 * quad]);
+          float4 v = make_float4(oacc[dt][0] * f, oacc[dt][1] * f, oacc[dt][2] * f, oacc[dt][3] * f);
+          if (w > 0) {
+            const float4 o = *dst;
+            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+          }
+          *dst = v;
+        }
+    }
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < nh * dv; c += 64 * NW) {
+    const int hh = c / dv, dd = c - hh * dv;
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) L += l_s[w][hh];
+    obase[c] = f2bf(L > 0.f ? o_s[hh * OP + dd] / L : 0.f);
+  }
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -100,29 +276,57 @@ using namespace k8sllm;
 extern "C" {
 
 int k8sllm_hy_latent_prep(void* proj, long stride, long T, int Q, int R, int dr, const float* qw, const float* kw,
-                          float eps, const int* positions, const float* freq, int nf, void* k_cache, void* v_cache,
-                          const int* slots, int bs, int f32, hipStream_t s) {
+                          float eps, const int* positions, const float* freq, int nf, void* k_cache, int kw_pitch,
+                          void* v_cache, const int* slots, int bs, int f32, hipStream_t s) {
   if (T <= 0) return 0;
-  if (2 * nf > dr) return -1;
+  if (2 * nf > dr || (k_cache != nullptr && kw_pitch < R + dr)) return -1;
   if (f32)
     hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(T), dim3(256), 0, s, (float*)proj, stride, Q, R, dr, qw, kw, eps,
-                       positions, freq, nf, (float*)k_cache, (float*)v_cache, slots, bs);
+                       positions, freq, nf, (float*)k_cache, kw_pitch, (float*)v_cache, slots, bs);
   else
     hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (bf16_t*)proj, stride, Q, R, dr, qw, kw,
-                       eps, positions, freq, nf, (bf16_t*)k_cache, (bf16_t*)v_cache, slots, bs);
+                       eps, positions, freq, nf, (bf16_t*)k_cache, kw_pitch, (bf16_t*)v_cache, slots, bs);
   return (int)hipGetLastError();
 }
 
 int k8sllm_hy_latent_queries(void* out, const void* q, long q_stride, const void* q_lat, long T, int H, int dn, int dr,
-                             int R, const int* positions, const float* freq, int nf, int f32, hipStream_t s) {
+                             int R, int w, const int* positions, const float* freq, int nf, int f32, hipStream_t s) {
   if (T <= 0) return 0;
-  if (2 * nf > dr) return -1;
+  if (2 * nf > dr || w < R + dr) return -1;
   if (f32)
     hipLaunchKernelGGL(latent_queries_kernel<float>, dim3(T), dim3(256), 0, s, (float*)out, (const float*)q, q_stride,
-                       (const float*)q_lat, T, H, dn, dr, R, positions, freq, nf);
+                       (const float*)q_lat, T, H, dn, dr, R, w, positions, freq, nf);
   else
     hipLaunchKernelGGL(latent_queries_kernel<bf16_t>, dim3(T), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)q,
-                       q_stride, (const bf16_t*)q_lat, T, H, dn, dr, R, positions, freq, nf);
+                       q_stride, (const bf16_t*)q_lat, T, H, dn, dr, R, w, positions, freq, nf);
+  return (int)hipGetLastError();
+}
+// Matrix-core latent attention (bf16): rows = T tokens, each at the position its segment (cu / ctx,
+// prompt chunks) or its sequence length (cu == nullptr, decoding) gives.  Returns 1 when the sizes
+// are not the kernel's (the caller then takes the any-size kernels): key rows padded to a multiple
+// of 32 (dkp), value width a multiple of 16, 16-token pages.
+int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const void* k_cache, const void* v_cache,
+                               const int* cu, const int* ctx, const int* seq_lens, const int* block_tables,
+                               int bt_stride, int S, long T, int H, int dkp, int dv, int bs, float scale, int window,
+                               const float* sinks, int split, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (bs != 16 || dkp % 32 || dv % 16 || dkp > 320 || dv > 256 || q_stride % 8) return 1;
+  const unsigned hgs = (unsigned)((H + 15) / 16);
+  // waves per (token, head group): a large step fills the chip with one; few rows (decoding) split
+  // the window over four
+  const int nw = split > 0 ? split : (T * hgs >= 2048 ? 1 : 4);
+  if (nw != 1 && nw != 4) return -1;
+  const dim3 grid((unsigned)T, hgs);
+#define K8SLLM_LA(KS, DT, NW)                                                                                          \
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KS, DT, NW>), grid, dim3(64 * NW), 0, s, (bf16_t*)out, (const bf16_t*)q,   \
+                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, seq_lens, block_tables,          \
+                     bt_stride, S, H, dkp, dv, scale, window, sinks)
+  if (dkp <= 128 && dv <= 128) {
+    if (nw == 1) K8SLLM_LA(4, 8, 1); else K8SLLM_LA(4, 8, 4);
+  } else {
+    if (nw == 1) K8SLLM_LA(10, 16, 1); else K8SLLM_LA(10, 16, 4);
+  }
+#undef K8SLLM_LA
   return (int)hipGetLastError();
 }
 }

@@ -300,8 +300,9 @@ def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw:
     """In place on the fused down-projections [T, q_rank | kv_rank | rot_dim] (or [T, q_rank] for a
     layer that reads another layer's cache): the query latent is RMS-normed (weight ``qw``); the
     key/value latent is RMS-normed (weight ``kw``) and the shared key part behind it is rotated by
-    its position (``freq``: rotary_freq); both go to the pages at ``slot_mapping`` - the key page row is [latent | rotated
-    part], the value page holds the latent once more, dim-major."""
+    its position (``freq``: rotary_freq); both go to the pages at ``slot_mapping`` - the key page
+    row is [latent | rotated part] (the page's rows may be wider: what lies behind is left as it is,
+    zero), the value page holds the latent once more, dim-major."""
     T = proj.shape[0]
     if not proj.is_cuda:
         q = proj[:, :q_rank].float()
@@ -316,7 +317,7 @@ def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw:
         ok = slot_mapping >= 0
         s = slot_mapping[ok].long()
         bs = k_cache.shape[1]
-        k_cache.view(-1, kv_rank + rot_dim)[s] = proj[ok, q_rank:]
+        k_cache.view(-1, k_cache.shape[2])[s, :kv_rank + rot_dim] = proj[ok, q_rank:]
         v_cache.view(-1, kv_rank, bs)[s // bs, :, s % bs] = c[ok]
         return
     native().latent_prep(proj, int(q_rank), int(kv_rank), int(rot_dim), qw, kw, float(eps), positions, freq,
@@ -324,18 +325,45 @@ def latent_prep(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, qw:
 
 
 def latent_queries(q: torch.Tensor, q_lat: torch.Tensor, H: int, dim: int, rot_dim: int, positions: torch.Tensor,
-                   freq: torch.Tensor) -> torch.Tensor:
-    """The queries against the latent cache: per head [q_lat | rotated part], [T, H * (R + rot_dim)].
+                   freq: torch.Tensor, pitch: int = 0) -> torch.Tensor:
+    """The queries against the latent cache: per head [q_lat | rotated part | zeros], [T, H * pitch]
+    (``pitch`` 0: R + rot_dim, no padding; else the key pages' row width).
     ``q`` [T, H * (dim + rot_dim)] are the up-projected queries (their last ``rot_dim`` entries per
     head are rotated by the position) and ``q_lat`` [H, T, R] the unrotated parts already
     multiplied into the latent space."""
     T, R = q.shape[0], q_lat.shape[2]
+    pitch = pitch or R + rot_dim
     if not q.is_cuda:
         qr = _rotate_half(q.view(T, H, dim + rot_dim)[..., dim:].float(), positions, freq).to(q.dtype)
-        return torch.cat([q_lat.transpose(0, 1), qr], -1).reshape(T, H * (R + rot_dim))
-    out = torch.empty(T, H * (R + rot_dim), dtype=q.dtype, device=q.device)
+        pad = torch.zeros(T, H, pitch - R - rot_dim, dtype=q.dtype)
+        return torch.cat([q_lat.transpose(0, 1), qr, pad], -1).reshape(T, H * pitch)
+    out = torch.empty(T, H * pitch, dtype=q.dtype, device=q.device)
     native().latent_queries(out, q, q_lat, int(H), int(dim), int(rot_dim), positions, freq)
     return out
+
+
+def latent_attention(qa: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                     H: int, scale: float, window: int, sinks: Optional[torch.Tensor], cu: Optional[torch.Tensor] = None,
+                     ctx: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None, fast: int = 1,
+                     split: int = 0) -> torch.Tensor:
+    """Attention of ``qa`` [T, H * pitch] (latent_queries) over the latent pages: every head reads
+    the one key stream ``k_cache`` [blocks, bs, pitch] and the one value stream ``v_cache`` [blocks, 1,
+    kv_rank, bs]; sliding window and learned sinks as in window_attention_*.  ``cu`` / ``ctx``: prompt
+    chunks (rows of segment s at positions ctx[s] ..); else ``seq_lens``: one row per sequence, at its
+    newest token.  Returns [T, H * kv_rank].  GPU, bf16, pitch a multiple of 32 up to 320 and kv_rank a
+    multiple of 16 up to 256 (``fast``): the matrix-core kernel, 16 heads of one token per tile
+    (``split``: waves that share a row's window, 1 or 4; 0: by the step's size); other sizes and fp32:
+    the any-size kernels with one shared key/value head."""
+    T, pitch, dv = qa.shape[0], k_cache.shape[2], v_cache.shape[2]
+    if qa.is_cuda and fast and qa.dtype == torch.bfloat16:
+        out = torch.empty(T, H * dv, dtype=qa.dtype, device=qa.device)
+        if native().latent_attention(out, qa, k_cache, v_cache, cu, ctx, seq_lens, block_tables, int(H), float(scale),
+                                     int(window), sinks, int(split)):
+            return out
+    args = (H, 1, pitch, dv, scale, window, True)
+    if cu is not None:
+        return window_attention_prefill(qa, k_cache, v_cache, cu, ctx, block_tables, *args, mfma=fast, sinks=sinks)
+    return window_attention_decode(qa, k_cache, v_cache, block_tables, seq_lens, *args, vec=bool(fast), sinks=sinks)
 
 
 # ---------------------------------------------------------------- Mamba-2

@@ -327,7 +327,8 @@ def test_latent_prep_and_queries(dt, Q, R, dr, nf):
     pos = torch.randint(0, 3000, (T,), generator=g, dtype=torch.int32)
     freq = H.rotary_freq(1000.0, 2 * nf)
     slots = _i32([17, 3, -1, 95, 64, 0, 33, 34, 35, 80, 15])
-    kc, vc = torch.zeros(nb, bs, R + dr, dtype=dt), torch.zeros(nb, 1, R, bs, dtype=dt)
+    pitch = (R + dr + 31) // 32 * 32  # wider than the row: the tail stays zero
+    kc, vc = torch.zeros(nb, bs, pitch, dtype=dt), torch.zeros(nb, 1, R, bs, dtype=dt)
     p_c, p_g, kg, vg = proj.clone(), proj.clone().cuda(), kc.clone().cuda(), vc.clone().cuda()
     H.latent_prep(p_c, Q, R, dr, qw, kw, 1e-6, pos, freq, kc, vc, slots)
     H.latent_prep(p_g, Q, R, dr, qw.cuda(), kw.cuda(), 1e-6, pos.cuda(), freq.cuda(), kg, vg, slots.cuda())
@@ -342,9 +343,13 @@ def test_latent_prep_and_queries(dt, Q, R, dr, nf):
     H.latent_prep(p2g, Q, R, dr, qw.cuda(), None, 1e-6, pos.cuda(), freq.cuda(), None, None, None)
     torch.testing.assert_close(p2g.cpu().float(), p2c.float(), **tol)
     q, ql = _r(g, T, H_ * (dn + dr), dt=dt), _r(g, H_, T, R, dt=dt)
-    want = H.latent_queries(q, ql, H_, dn, dr, pos, freq)
-    got = H.latent_queries(q.cuda(), ql.cuda(), H_, dn, dr, pos.cuda(), freq.cuda())
-    torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+    for pt in (0, pitch):
+        want = H.latent_queries(q, ql, H_, dn, dr, pos, freq, pt)
+        got = H.latent_queries(q.cuda(), ql.cuda(), H_, dn, dr, pos.cuda(), freq.cuda(), pt)
+        assert want.shape == (T, H_ * (pt or R + dr))
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol)
+    assert float(kc[..., R + dr:].abs().max() if pitch > R + dr else 0.0) == 0.0
+    assert float(kg[..., R + dr:].abs().max() if pitch > R + dr else 0.0) == 0.0
 
 
 @pytest.mark.parametrize("dt", DT)
@@ -395,3 +400,33 @@ def test_router_over_all_and_gelu_experts(dt):
             got = H.moe_experts(h.cuda(), ids_g, w_g, w1.cuda(), w2.cuda(), sh.cuda() if sh is not None else None, None,
                                 act="gelu", mfma=mfma)
             torch.testing.assert_close(got.cpu(), want, **_tol(dt))
+
+
+@pytest.mark.parametrize("Hq,pitch,dv", [(8, 128, 112), (16, 320, 256), (20, 64, 48), (3, 96, 16), (1, 32, 32)])
+@pytest.mark.parametrize("window", [24, 0, 300])
+def test_latent_attention_matrix_core(Hq, pitch, dv, window):
+    """The head-packed matrix-core kernel (one wave per row, and the window split over four waves)
+    against the torch form: prompt chunks with context, single rows, padding rows, partial head groups."""
+    dt = torch.bfloat16
+    g = _g(17)
+    lens, chunk = [350, 9, 33, 70], [20, 9, 2, 70]
+    kc, vc, bt = _paged(g, dt, lens, Hq, 1, pitch, dv, nb=60)
+    sinks = _r(g, Hq, s=1.5)
+    T = sum(chunk)
+    qa = _r(g, T, Hq * pitch, s=0.25, dt=dt)
+    cu = _i32([0, 20, 29, 31, 101])
+    ctx = _i32([n - c for n, c in zip(lens, chunk)])
+    want = H.latent_attention(qa, kc, vc, bt, Hq, 0.2, window, sinks, cu=cu, ctx=ctx)
+    dev = lambda *ts: [t.cuda() for t in ts]  # noqa: E731
+    for split in (1, 4, 0):
+        got = H.latent_attention(*dev(qa, kc, vc, bt), Hq, 0.2, window, sinks.cuda(), cu=cu.cuda(), ctx=ctx.cuda(),
+                                 split=split)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+    q1 = _r(g, 5, Hq * pitch, s=0.25, dt=dt)
+    sl = _i32(lens + [0])  # the last row is a padding row
+    bt5 = torch.cat([bt, bt[:1]])
+    want = H.latent_attention(q1, kc, vc, bt5, Hq, 0.2, window, sinks, seq_lens=sl)
+    for split in (1, 4, 0):
+        got = H.latent_attention(*dev(q1, kc, vc, bt5), Hq, 0.2, window, sinks.cuda(), seq_lens=sl.cuda(), split=split)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+        assert float(got[4].abs().max()) == 0.0
