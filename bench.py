@@ -17,8 +17,9 @@ Modes (``--mode``):
   at ``--rate`` queries/s; reports TTFT / TPOT / latency percentiles (mixed prefill+decode steps
   at work).
 * ``latency`` - batch 1: one query at a time; a step = one query.
-* ``arch`` - not the headline: prefill and decode tokens/s of the Dunesun layer-list design beside
-  a Mixtral-style model of equal layer sizes (engine/arch_bench.py), one GPU, random weights.
+* ``arch`` - not the headline: prefill and decode tokens/s of a layer-list design beside its closest
+  existing model at equal layer sizes (engine/arch_bench.py; ``--arch-design dunesun``: beside a
+  Mixtral-style model, ``kisutar``: beside an all-attention Dunesun model), one GPU, random weights.
 ``--production``: the server runs with the reference's timeouts (15 s write, 30 s llm.timeout)
 instead of the bench's 600 s; answers that reach the deadline come back truncated
 (finish_reason "deadline") and overload as 503 - both are counted in the JSON line.
@@ -69,6 +70,8 @@ def parse(argv=None):
     ap.add_argument("--arch-seqs", type=int, default=4, help="arch: prompts in the prefill step")
     ap.add_argument("--arch-window", type=int, default=1024, help="arch: the Dunesun attention layers' window")
     ap.add_argument("--arch-which", choices=["both", "new", "ref"], default="both")
+    ap.add_argument("--arch-design", choices=["dunesun", "kisutar"], default="dunesun",
+                    help="arch: the layer-list design to measure beside its closest existing model")
     ap.add_argument("--rate", type=float, default=16.0, help="poisson: arrivals per second per replica")
     ap.add_argument("--production", action="store_true",
                     help="reference server timeouts (15 s write / 30 s llm): deadline truncation + 503s")

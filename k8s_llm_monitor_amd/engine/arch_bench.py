@@ -1,8 +1,10 @@
-"""Prefill and decode throughput of the Dunesun design beside the closest existing model
-(Mixtral-style: attention + routed experts in every layer) at equal layer sizes, random weights,
-one GPU (``python bench.py --mode arch``).  Both models run through the same ModelRunner step
-functions the engine uses: one prefill step of ``seqs`` whole prompts, then decode steps of
-``batch`` sequences (hipGraph replay where the model's decode is captured)."""
+"""Prefill and decode throughput of a layer-list design beside the closest existing model at equal
+layer sizes, random weights, one GPU (``python bench.py --mode arch [--arch-design NAME]``):
+Dunesun beside a Mixtral-style model (attention + routed experts in every layer); Kisutar beside
+an all-attention Dunesun model (windowed attention with sinks, fp32 residual stream, routed experts
+with a shared expert in every layer - the same kernels family).  Both models run through the same
+ModelRunner step functions the engine uses: one prefill step of ``seqs`` whole prompts, then decode
+steps of ``batch`` sequences (hipGraph replay where the model's decode is captured)."""
 from __future__ import annotations
 
 import json
@@ -10,7 +12,7 @@ import time
 
 import torch
 
-from ..models.config import HybridConfig, LayerSpec, ModelConfig, MoESpec
+from ..models.config import DenseSpec, HybridConfig, LayerSpec, ModelConfig, MoESpec
 from ..models.registry import build_model
 from .block_manager import BlockManager
 from .runner import ModelRunner, RunnerConfig
@@ -36,6 +38,39 @@ def _pair(size: str, window: int) -> tuple:
                       n_kv_heads=G, head_dim=D, ffn_dim=ff, max_position=8192, rope_theta=1e6, n_experts=E,
                       top_k_experts=K, bos_id=1, eos_ids=(2,))
     return hy, ref
+
+
+# Kisutar: (name, width, heads, unrotated dim, rotated dim, value dim, q rank, kv rank, experts, top, expert ff,
+#           shared ff, dense ff, layers); the reference gets the same width, heads, head size dim + rot, experts
+KISUTAR_SIZES = {
+    "s": ("d1024", 1024, 8, 96, 32, 128, 384, 128, 8, 2, 1024, 1024, 4096, 4),
+    "m": ("d2048", 2048, 16, 96, 32, 128, 768, 256, 8, 2, 2048, 2048, 8192, 4),
+    "l": ("d4096", 4096, 32, 96, 32, 128, 1536, 256, 8, 2, 3584, 3584, 14336, 2),
+}
+
+
+def _kisutar_pair(size: str, window: int) -> tuple:
+    """Kisutar (dense and routed layers alternating, the second half of the layers reading the pages
+    of the last layer before them that has its own) and an all-attention Dunesun model of equal
+    width, heads, head size and experts."""
+    name, d, H, dn, dr, dv, Q, R, E, K, ff, fs, fd, L = KISUTAR_SIZES[size]
+    own = max(1, L // 2)
+
+    def lat(i):
+        m = {"heads": H, "dim": dn, "rot_dim": dr, "vdim": dv, "q_rank": Q, "kv_rank": R, "mask.size": window,
+             "scale": (dn + dr) ** -0.5, "rot.base": 10000.0, "rot.dims": dr}
+        if i >= own:
+            m["kv_from"] = own - 1
+        return LayerSpec("latent_attention", tuple(sorted(m.items())), DenseSpec(fd) if i % 2 == 0 else MoESpec(E, K, ff, fs))
+
+    new = HybridConfig(name=f"kisutar-{name}", arch="kisutar", vocab_size=32000, d_model=d,
+                       layers=tuple(lat(i) for i in range(L)), max_position=8192, norm_eps=1e-6)
+    D = dn + dr
+    att = LayerSpec("attention", tuple(sorted({"heads": H, "kv_heads": max(1, H // 4), "dim": D, "vdim": D, "mask.size": window,
+                                               "scale": D ** -0.5}.items())), MoESpec(E, K, ff, fs))
+    ref = HybridConfig(name=f"dunesun-attn-{name}", arch="dunesun", vocab_size=32000, d_model=d,
+                       layers=tuple(att for _ in range(L)), max_position=8192)
+    return new, ref
 
 
 def _measure(cfg, seqs: int, prompt: int, batch: int, steps: int, warmup: int, graphs: bool) -> dict:
@@ -106,7 +141,7 @@ def run(a) -> None:
     """``a``: bench.py's parsed arguments (arch_sizes, arch_prompt, arch_seqs, batch, steps, warmup)."""
     rows = []
     for size in a.arch_sizes.split(","):
-        hy, ref = _pair(size, a.arch_window)
+        hy, ref = (_kisutar_pair if getattr(a, "arch_design", "dunesun") == "kisutar" else _pair)(size, a.arch_window)
         for cfg in ((hy, ref) if a.arch_which == "both" else ((hy,) if a.arch_which == "new" else (ref,))):
             r = _measure(cfg, a.arch_seqs, a.arch_prompt, a.batch, a.steps, a.warmup, not a.no_graphs)
             r["size"] = size
@@ -114,7 +149,7 @@ def run(a) -> None:
             print(json.dumps(r), flush=True)
     line = {"metric": "arch_compare_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
             "dtype": "bf16", "data": "synthetic", "higher_is_better": True,
-            "config": {"prompt": a.arch_prompt, "prefill_seqs": a.arch_seqs, "decode_batch": a.batch,
+            "config": {"design": getattr(a, "arch_design", "dunesun"), "prompt": a.arch_prompt, "prefill_seqs": a.arch_seqs, "decode_batch": a.batch,
                        "window": a.arch_window}, "rows": rows}
     print(json.dumps(line), flush=True)
     if a.out:

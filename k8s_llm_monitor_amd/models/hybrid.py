@@ -317,6 +317,8 @@ class PlainRoutedFFN:
             raise ValueError(f"{prefix}: top {self.K} of {self.E} experts")
         s, s2 = 1.0 / math.sqrt(d), 1.0 / math.sqrt(self.ff)
         self.il = False
+        # large bf16 steps of such experts run on the Mixtral path's tile GEMM (ops.hybrid.moe_experts)
+        self.tile = p.device.type == "cuda" and p.dtype == torch.bfloat16 and self.ff % 256 == 0 and d % 256 == 0
         self.w1 = torch.stack([p.get(f"{prefix}e{e}.up", (self.ff, d), s) for e in range(self.E)])
         self.w2 = torch.stack([p.get(f"{prefix}e{e}.down", (d, self.ff), s2) for e in range(self.E)])
         self.wr = p.get(prefix + "router", (self.E, d), 2 * s, small=True)
@@ -408,7 +410,8 @@ class HybridLM:
         self.unused = sorted(set(weights.keys()) - p.used) if weights is not None else []
         self.has_state = self.shifted or any(m.kind == "mamba2" for m in self.mixers)
         # large steps of such layers run on the Mixtral path's tile GEMM (extension _k8sllm_ops)
-        self.uses_tile_gemm = any(f is not None and getattr(f, "il", False) for f in self.ffns)
+        self.uses_tile_gemm = any(f is not None and (getattr(f, "il", False) or getattr(f, "tile", False))
+                                  for f in self.ffns)
         self.layer_probe = None  # a list: forward() appends the residual stream after every run
 
     # ------------------------------------------------------------------ engine interface

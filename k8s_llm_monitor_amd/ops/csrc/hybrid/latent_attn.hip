@@ -112,53 +112,81 @@ __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out
 // only parallel axis of a row) and merge their (maximum, denominator, output) through LDS: the common
 // maximum first, then the outputs summed wave after wave into one buffer.  Only wave 0 starts from
 // the sink.  Scores, weights and sums are fp32, base-2 exponentials (the scale carries log2 e).
+// QT consecutive tokens of a prompt chunk share a wave's key and value fragments (their windows
+// differ by one key at each end).
 // KS_MAX / DT_MAX bound the key width / 32 and the value width / 16 (register arrays); the real
 // widths are run-time (wave-uniform guards).  cu == nullptr: one row per sequence at seq_lens - 1.
-template <int KS_MAX, int DT_MAX, int NW>
+template <int KS_MAX, int DT_MAX, int NW, int QT, bool DB>
 __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
     const int* __restrict__ seq_lens, const int* __restrict__ block_tables, int bt_stride, int S, int H, int dkp,
     int dv, float scale, int window, const float* __restrict__ sinks) {
+  static_assert(NW == 1 || QT == 1, "the window is split over waves only for single tokens");
   constexpr int OP = DT_MAX * 16 + 4;  // LDS row pitch of the merge buffer (floats)
   __shared__ __attribute__((aligned(16))) float o_s[NW > 1 ? 16 * OP : 4];
   __shared__ float m_s[NW > 1 ? NW : 1][16];
   __shared__ float l_s[NW > 1 ? NW : 1][16];
   const float sc2 = scale * 1.44269504088896341f;
-  const int row = blockIdx.x, hg = blockIdx.y;
+  // Workgroups go to the 8 XCDs in turn (each with an L2 of its own): give every XCD one contiguous
+  // eighth of the (token group, head group) list, so that the windows its waves read overlap in ITS L2
+  const int nwg = gridDim.x * gridDim.y, lin = blockIdx.y * gridDim.x + blockIdx.x;
+  const int xcd = lin & 7, glin = xcd * (nwg >> 3) + min(xcd, nwg & 7) + (lin >> 3);  // XCD x: workgroups x, x + 8, ..
+  const int hg = glin % (int)gridDim.y, bx = glin / (int)gridDim.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c16 = lane & 15, quad = lane >> 4;
-  int s, p;
+  // this workgroup's tokens: QT consecutive rows of one segment (token groups are numbered segment
+  // by segment), or one sequence's newest token
+  int s = 0, row0, p0, nt = 1;
   if (cu != nullptr) {
-    s = find_segment(cu, S, row);
-    p = ctx[s] + row - cu[s];
+    if (QT == 1) {
+      row0 = bx;
+      s = find_segment(cu, S, row0);
+      p0 = ctx[s] + row0 - cu[s];
+    } else {
+      int g = bx, n = 0;
+      for (; s < S; ++s) {
+        n = cu[s + 1] - cu[s];
+        const int ng = (n + QT - 1) / QT;
+        if (g < ng) break;
+        g -= ng;
+      }
+      if (s >= S) return;
+      row0 = cu[s] + g * QT;
+      nt = min(QT, n - g * QT);
+      p0 = ctx[s] + g * QT;
+    }
   } else {
-    s = row;
-    p = seq_lens[row] - 1;
+    s = row0 = bx;
+    p0 = seq_lens[row0] - 1;
   }
   const int nh = min(16, H - hg * 16);
-  bf16_t* obase = out + ((long)row * H + hg * 16) * dv;
-  if (p < 0) {  // padding row of a decode bucket
+  bf16_t* obase = out + ((long)row0 * H + hg * 16) * dv;
+  if (p0 < 0) {  // padding row of a decode bucket
     for (int c = threadIdx.x; c < nh * dv; c += 64 * NW) obase[c] = 0;
     return;
   }
   const int nks = dkp >> 5, ndt = dv >> 4;
   const int head = hg * 16 + min(c16, nh - 1);
   const int* bt = block_tables + (long)s * bt_stride;
-  const int lo = window > 0 ? max(0, p - window + 1) : 0, hi = p + 1;
-  bf16x8 qf[KS_MAX];
-  {
-    const bf16_t* qrow = q + (long)row * q_stride + (long)head * dkp + 8 * quad;
+  // token t of the group sits at position p0 + t and sees keys lo_t .. p0 + t
+  const int lo = window > 0 ? max(0, p0 - window + 1) : 0, hi = p0 + nt;
+  bf16x8 qf[QT][KS_MAX];
+  f32x4 oacc[QT][DT_MAX];
+  float m[QT], l[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const bf16_t* qrow = q + (long)(row0 + min(t, nt - 1)) * q_stride + (long)head * dkp + 8 * quad;
 #pragma unroll
     for (int ks = 0; ks < KS_MAX; ++ks)
-      if (ks < nks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
-  }
-  f32x4 oacc[DT_MAX];
+      if (ks < nks) qf[t][ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
 #pragma unroll
-  for (int dt = 0; dt < DT_MAX; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  if (wave == 0) {
-    m = sinks != nullptr ? sinks[head] * 1.44269504088896341f : 0.f;
-    l = 1.f;
+    for (int dt = 0; dt < DT_MAX; ++dt) oacc[t][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+    if (wave == 0) {
+      m[t] = sinks != nullptr ? sinks[head] * 1.44269504088896341f : 0.f;
+      l[t] = 1.f;
+    }
   }
   const bf16_t* kbase = k_cache + 8 * quad;
   const bf16_t* vbase = v_cache + (long)c16 * 16 + 4 * quad;
@@ -177,80 +205,97 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
     for (int dt = 0; dt < DT_MAX; ++dt)
       if (dt < ndt) vf_n[dt] = *reinterpret_cast<const s16x4*>(vpg + dt * 256);
   };
-  if (jfirst < hi) issue(jfirst);
+  // DB: the next tile's fragments are in flight while this one is computed (one wave per SIMD hides
+  // its own latency); else fewer registers and more waves per SIMD hide each other's
+  if (DB && jfirst < hi) issue(jfirst);
   for (int j0 = jfirst; j0 < hi; j0 += 16 * NW) {
     bf16x8 kf[KS_MAX];
     s16x4 vf[DT_MAX];
+    if (!DB) issue(j0);
 #pragma unroll
     for (int ks = 0; ks < KS_MAX; ++ks) kf[ks] = kf_n[ks];
 #pragma unroll
     for (int dt = 0; dt < DT_MAX; ++dt) vf[dt] = vf_n[dt];
-    if (j0 + 16 * NW < hi) issue(j0 + 16 * NW);
-    f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (DB && j0 + 16 * NW < hi) issue(j0 + 16 * NW);
+    s16x4 pb[QT];
+    float alpha[QT];
+    bool rescale[QT];
 #pragma unroll
-    for (int ks = 0; ks < KS_MAX; ++ks)
-      if (ks < nks) sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], sacc, 0, 0, 0);
-    float sv[4], tmax = -INFINITY;
+    for (int t = 0; t < QT; ++t) {
+      f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, head c16
-      const int j = j0 + 4 * quad + i;
-      sv[i] = (j >= lo && j < hi) ? sacc[i] * sc2 : -INFINITY;
-      tmax = fmaxf(tmax, sv[i]);
+      for (int ks = 0; ks < KS_MAX; ++ks)
+        if (ks < nks) sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[t][ks], sacc, 0, 0, 0);
+      const int pt = p0 + t, lot = window > 0 ? max(0, pt - window + 1) : 0;
+      float sv[4], tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, head c16
+        const int j = j0 + 4 * quad + i;
+        sv[i] = (t < nt && j >= lot && j <= pt) ? sacc[i] * sc2 : -INFINITY;
+        tmax = fmaxf(tmax, sv[i]);
+      }
+      tmax = xor32_max_f(xor16_max(tmax));
+      const float mn = fmaxf(m[t], tmax);
+      // a tile may hold no live key of token t (QT > 1: the window's first or last tile): nothing moves
+      alpha[t] = (m[t] == -INFINITY || mn == -INFINITY) ? (mn == -INFINITY ? 1.f : 0.f) : __builtin_amdgcn_exp2f(m[t] - mn);
+      float ps = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = sv[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sv[i] - mn);
+        ps += pv;
+        pb[t][i] = (short)f2bf(pv);
+      }
+      ps = xor32_sum_f(xor16_sum(ps));
+      l[t] = l[t] * alpha[t] + ps;
+      m[t] = mn;
+      rescale[t] = __any(alpha[t] != 1.f);
     }
-    tmax = xor32_max_f(xor16_max(tmax));
-    const float mn = fmaxf(m, tmax);  // the tile holds at least one live key
-    const float alpha = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - mn);
-    float ps = 0.f;
-    s16x4 pb;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float pv = sv[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sv[i] - mn);
-      ps += pv;
-      pb[i] = (short)f2bf(pv);
-    }
-    ps = xor32_sum_f(xor16_sum(ps));
-    l = l * alpha + ps;
-    m = mn;
-    const bool rescale = __any(alpha != 1.f);
 #pragma unroll
     for (int dt = 0; dt < DT_MAX; ++dt)
       if (dt < ndt) {
-        if (rescale) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) oacc[dt][i] *= alpha;
+        for (int t = 0; t < QT; ++t) {
+          if (rescale[t]) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
+          }
+          oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[dt], pb[t], oacc[t][dt], 0, 0, 0);
         }
-        oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[dt], pb, oacc[dt], 0, 0, 0);
       }
   }
-  // oacc[dt][i] = O[head c16][d = 16 dt + 4 quad + i]
+  // oacc[t][dt][i] = O[token t][head c16][d = 16 dt + 4 quad + i]
   if (NW == 1) {
     if (c16 >= nh) return;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    bf16_t* orow = obase + (long)c16 * dv;
 #pragma unroll
-    for (int dt = 0; dt < DT_MAX; ++dt)
-      if (dt < ndt) {
-        uint2 w;
-        w.x = pack2(oacc[dt][0] * inv, oacc[dt][1] * inv);
-        w.y = pack2(oacc[dt][2] * inv, oacc[dt][3] * inv);
-        *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * quad) = w;
-      }
+    for (int t = 0; t < QT; ++t) {
+      if (t >= nt) break;
+      const float inv = l[t] > 0.f ? 1.f / l[t] : 0.f;
+      bf16_t* orow = obase + ((long)t * H + c16) * dv;
+#pragma unroll
+      for (int dt = 0; dt < DT_MAX; ++dt)
+        if (dt < ndt) {
+          uint2 w;
+          w.x = pack2(oacc[t][dt][0] * inv, oacc[t][dt][1] * inv);
+          w.y = pack2(oacc[t][dt][2] * inv, oacc[t][dt][3] * inv);
+          *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * quad) = w;
+        }
+    }
     return;
   }
-  if (quad == 0) m_s[wave][c16] = m;
+  if (quad == 0) m_s[wave][c16] = m[0];
   __syncthreads();
   float M = -INFINITY;
 #pragma unroll
   for (int w = 0; w < NW; ++w) M = fmaxf(M, m_s[w][c16]);  // wave 0's is finite (the sink)
-  const float f = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);
-  if (quad == 0) l_s[wave][c16] = l * f;
+  const float f = m[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[0] - M);
+  if (quad == 0) l_s[wave][c16] = l[0] * f;
   for (int w = 0; w < NW; ++w) {
     if (wave == w) {
 #pragma unroll
       for (int dt = 0; dt < DT_MAX; ++dt)
         if (dt < ndt) {
           float4* dst = reinterpret_cast<float4*>(&o_s[c16 * OP + 16 * dt + 4 * quad]);
-          float4 v = make_float4(oacc[dt][0] * f, oacc[dt][1] * f, oacc[dt][2] * f, oacc[dt][3] * f);
+          float4 v = make_float4(oacc[0][dt][0] * f, oacc[0][dt][1] * f, oacc[0][dt][2] * f, oacc[0][dt][3] * f);
           if (w > 0) {
             const float4 o = *dst;
             v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
@@ -312,20 +357,32 @@ int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const vo
   if (T <= 0) return 0;
   if (bs != 16 || dkp % 32 || dv % 16 || dkp > 320 || dv > 256 || q_stride % 8) return 1;
   const unsigned hgs = (unsigned)((H + 15) / 16);
-  // waves per (token, head group): a large step fills the chip with one; few rows (decoding) split
-  // the window over four
-  const int nw = split > 0 ? split : (T * hgs >= 2048 ? 1 : 4);
-  if (nw != 1 && nw != 4) return -1;
-  const dim3 grid((unsigned)T, hgs);
-#define K8SLLM_LA(KS, DT, NW)                                                                                          \
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<KS, DT, NW>), grid, dim3(64 * NW), 0, s, (bf16_t*)out, (const bf16_t*)q,   \
-                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, seq_lens, block_tables,          \
-                     bt_stride, S, H, dkp, dv, scale, window, sinks)
-  if (dkp <= 128 && dv <= 128) {
-    if (nw == 1) K8SLLM_LA(4, 8, 1); else K8SLLM_LA(4, 8, 4);
-  } else {
-    if (nw == 1) K8SLLM_LA(10, 16, 1); else K8SLLM_LA(10, 16, 4);
-  }
+  // split 1 / 4 force that many waves with one token each (tests, measurements); 2: two tokens per wave
+  // prompt chunks: two tokens per wave, no register double buffer (two waves per SIMD hide each
+  // other's loads better than one wave hides its own: measured); few rows: eight waves per token.
+  // split: 1 / 2 tokens per wave, 4 / 8 waves per token; + 16: with the register double buffer
+  const bool big = T * hgs >= 2048;
+  const bool db = split >= 16;
+  if (db) split -= 16;
+  if (split != 0 && split != 1 && split != 2 && split != 4 && split != 8) return -1;
+  const int nw = split == 4 || split == 8 ? split : ((split == 1 || split == 2 || big) ? 1 : 8);
+  const int qt = (cu != nullptr && nw == 1 && split != 1) ? 2 : 1;
+  const dim3 grid((unsigned)(qt == 1 ? T : T / qt + S), hgs);
+#define K8SLLM_LA(KS, DT, NW, QT, DB)                                                                                  \
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KS, DT, NW, QT, DB>), grid, dim3(64 * NW), 0, s, (bf16_t*)out,            \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, seq_lens,     \
+                     block_tables, bt_stride, S, H, dkp, dv, scale, window, sinks)
+#define K8SLLM_LAS(KS, DT)                                            \
+  if (nw == 8) K8SLLM_LA(KS, DT, 8, 1, false);                        \
+  else if (nw == 4 && db) K8SLLM_LA(KS, DT, 4, 1, true);              \
+  else if (nw == 4) K8SLLM_LA(KS, DT, 4, 1, false);                   \
+  else if (qt == 2 && db) K8SLLM_LA(KS, DT, 1, 2, true);              \
+  else if (qt == 2) K8SLLM_LA(KS, DT, 1, 2, false);                   \
+  else if (db) K8SLLM_LA(KS, DT, 1, 1, true);                         \
+  else K8SLLM_LA(KS, DT, 1, 1, false)
+  if (dkp <= 128 && dv <= 128) { K8SLLM_LAS(4, 8); }
+  else { K8SLLM_LAS(10, 16); }
+#undef K8SLLM_LAS
 #undef K8SLLM_LA
   return (int)hipGetLastError();
 }

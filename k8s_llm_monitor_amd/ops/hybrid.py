@@ -352,7 +352,8 @@ def latent_attention(qa: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     chunks (rows of segment s at positions ctx[s] ..); else ``seq_lens``: one row per sequence, at its
     newest token.  Returns [T, H * kv_rank].  GPU, bf16, pitch a multiple of 32 up to 320 and kv_rank a
     multiple of 16 up to 256 (``fast``): the matrix-core kernel, 16 heads of one token per tile
-    (``split``: waves that share a row's window, 1 or 4; 0: by the step's size); other sizes and fp32:
+    (``split`` 1: one wave per token, 2: two tokens of a chunk per wave, 4 / 8: that many waves share
+    a token's window, + 16: with the register double buffer; 0: by the step's size); other sizes and fp32:
     the any-size kernels with one shared key/value head."""
     T, pitch, dv = qa.shape[0], k_cache.shape[2], v_cache.shape[2]
     if qa.is_cuda and fast and qa.dtype == torch.bfloat16:
@@ -501,7 +502,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
     run as ONE grouped launch each over the sorted rows (SwiGLU in the first epilogue); no host
     synchronisation.  bf16: matrix-core kernels - 16-row tiles with the rows gathered on load
     (decode, small steps), or from TILE_MIN_ROWS sorted rows of an ``il`` layer the prefill tile
-    GEMM of the Mixtral path; fp32 (and K not a multiple of 32): the 64 x 64 fp32 tile kernel."""
+    GEMM of the Mixtral path (ungated experts whose widths are multiples of 256 take it too, with
+    the GELU as a launch between); fp32 (and K not a multiple of 32): the 64 x 64 fp32 tile kernel."""
     T, d = h.shape
     E, K = w13.shape[0], ids.shape[1]
     ff = w2.shape[2]
@@ -530,7 +532,13 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w13: torc
     inv_idx = torch.empty(n, dtype=torch.int32, device=h.device)
     ext.moe_align(ids, E, offsets, sorted_idx, inv_idx)
     code = {"swiglu": 1, "gelu": 2}[act]
-    if il and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16:
+    if act == "gelu" and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16 and ff % 256 == 0 and d % 256 == 0:
+        from .. import ops  # large steps of plain experts: the prefill tile GEMM twice, GELU between
+
+        xs = ops.gather_rows(h, sorted_idx, K)
+        a = activation(ops.moe_grouped_gemm(xs, w13, offsets, zero_fill=False), "gelu")
+        ys = ops.moe_grouped_gemm(a, w2, offsets, zero_fill=False)
+    elif il and n >= TILE_MIN_ROWS and h.dtype == torch.bfloat16:
         from .. import ops  # the Mixtral path's kernels (_k8sllm_ops)
 
         xs = ops.gather_rows(h, sorted_idx, K)

@@ -405,7 +405,8 @@ def test_router_over_all_and_gelu_experts(dt):
 @pytest.mark.parametrize("Hq,pitch,dv", [(8, 128, 112), (16, 320, 256), (20, 64, 48), (3, 96, 16), (1, 32, 32)])
 @pytest.mark.parametrize("window", [24, 0, 300])
 def test_latent_attention_matrix_core(Hq, pitch, dv, window):
-    """The head-packed matrix-core kernel (one wave per row, and the window split over four waves)
+    """The head-packed matrix-core kernel (one wave per row, two rows per wave, the window split
+    over four or eight waves, with and without the register double buffer)
     against the torch form: prompt chunks with context, single rows, padding rows, partial head groups."""
     dt = torch.bfloat16
     g = _g(17)
@@ -418,7 +419,7 @@ def test_latent_attention_matrix_core(Hq, pitch, dv, window):
     ctx = _i32([n - c for n, c in zip(lens, chunk)])
     want = H.latent_attention(qa, kc, vc, bt, Hq, 0.2, window, sinks, cu=cu, ctx=ctx)
     dev = lambda *ts: [t.cuda() for t in ts]  # noqa: E731
-    for split in (1, 4, 0):
+    for split in (1, 2, 4, 8, 17, 18, 0):
         got = H.latent_attention(*dev(qa, kc, vc, bt), Hq, 0.2, window, sinks.cuda(), cu=cu.cuda(), ctx=ctx.cuda(),
                                  split=split)
         torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
@@ -426,7 +427,22 @@ def test_latent_attention_matrix_core(Hq, pitch, dv, window):
     sl = _i32(lens + [0])  # the last row is a padding row
     bt5 = torch.cat([bt, bt[:1]])
     want = H.latent_attention(q1, kc, vc, bt5, Hq, 0.2, window, sinks, seq_lens=sl)
-    for split in (1, 4, 0):
+    for split in (1, 4, 8, 20, 0):
         got = H.latent_attention(*dev(q1, kc, vc, bt5), Hq, 0.2, window, sinks.cuda(), seq_lens=sl.cuda(), split=split)
         torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
         assert float(got[4].abs().max()) == 0.0
+
+
+def test_gelu_experts_on_the_tile_gemm():
+    """Widths that are multiples of 256 and a large step: the ungated experts go through the
+    prefill tile GEMM and agree with the 16-row kernel and the torch form."""
+    dt = torch.bfloat16
+    g = _g(18)
+    T, d, E, K, ff = 700, 256, 4, 2, 512  # 1400 routed rows
+    h = _r(g, T, d, dt=dt)
+    wr = _r(g, E, d, s=0.3)
+    ids, wts, _ = H.moe_router(h, wr, None, E, K, over_all=True)
+    w1, w2 = _r(g, E, ff, d, s=d ** -0.5, dt=dt), _r(g, E, d, ff, s=ff ** -0.5, dt=dt)
+    want = H.moe_experts(h, ids, wts, w1, w2, None, None, act="gelu")
+    got = H.moe_experts(h.cuda(), ids.cuda(), wts.cuda(), w1.cuda(), w2.cuda(), None, None, act="gelu")
+    torch.testing.assert_close(got.cpu(), want, **_tol(dt))
