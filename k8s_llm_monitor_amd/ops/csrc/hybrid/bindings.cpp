@@ -420,7 +420,6 @@ void depth_mix(Tensor stack, int64_t n, OptT addend, Tensor coef) {
   TORCH_CHECK(stack.dim() == 3 && n >= 0 && n + 1 < stack.size(0) && coef.numel() == n + 1 && n < 256,
               "depth_mix: stack [L, T, d], coef [n + 1], n + 1 < L");
   const int64_t plane = stack.size(1) * stack.size(2);
-  TORCH_CHECK(plane % 4 == 0, "depth_mix: T * d must be a multiple of 4");
   const int adt = any_dt(addend, plane, "addend");
   check(k8sllm_hy_depth_mix(stack.data_ptr<float>(), plane, (int)n, adt ? addend->data_ptr() : nullptr, adt,
                             coef.data_ptr<float>(), cur()),

@@ -215,6 +215,22 @@ __global__ __launch_bounds__(256) void depth_mix_kernel(float* __restrict__ stac
   *reinterpret_cast<float4*>(stack + (long)(n + 1) * plane + i) = acc;
 }
 
+// any T * d: one element per thread
+__global__ __launch_bounds__(256) void depth_mix_scalar_kernel(float* __restrict__ stack, long plane, int n,
+                                                               const void* __restrict__ addend, int adt,
+                                                               const float* __restrict__ coef) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= plane) return;
+  float top = stack[(long)n * plane + i];
+  if (adt) {
+    top += ld_any(addend, adt, i);
+    stack[(long)n * plane + i] = top;
+  }
+  float acc = 0.f;
+  for (int j = 0; j < n; ++j) acc += coef[j] * stack[(long)j * plane + i];
+  stack[(long)(n + 1) * plane + i] = acc + coef[n] * top;
+}
+
 // KIND 0: erf GELU, 1: tanh GELU, 2: xIELU (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below)
 template <int KIND>
 __device__ __forceinline__ float act_f(float z, float a, float b) {
@@ -309,11 +325,16 @@ int k8sllm_hy_norm_shift(void* out, const float* x, const float* w, const float*
   return (int)hipGetLastError();
 }
 
-// plane = T * d (a multiple of 4)
+// plane = T * d
 int k8sllm_hy_depth_mix(float* stack, long plane, int n, const void* addend, int adt, const float* coef,
                         hipStream_t s) {
   if (plane <= 0) return 0;
-  if (n < 0 || n >= kMaxDepth || (plane & 3)) return -1;
+  if (n < 0 || n >= kMaxDepth) return -1;
+  if (plane & 3) {
+    hipLaunchKernelGGL(depth_mix_scalar_kernel, dim3((unsigned)((plane + 255) / 256)), dim3(256), 0, s, stack, plane, n,
+                       addend, adt, coef);
+    return (int)hipGetLastError();
+  }
   hipLaunchKernelGGL(depth_mix_kernel, dim3((unsigned)((plane / 4 + 255) / 256)), dim3(256), 0, s, stack, plane, n,
                      addend, adt, coef);
   return (int)hipGetLastError();

@@ -11,8 +11,10 @@
 
 namespace k8sllm {
 
-constexpr int kMaxVC = 4;  // output dims per lane: dv <= 64 * kMaxVC
+constexpr int kMaxVC = 4;  // output dims per lane of the vector decode kernel: dv <= 64 * kMaxVC
 constexpr int kMaxDK = 512;
+constexpr int kGenVC = 8;  // the any-size kernels: dv <= 64 * kGenVC, dk <= kGenDK
+constexpr int kGenDK = 1024;
 
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_cache_kernel(T* __restrict__ qkv, long stride,
@@ -55,9 +57,9 @@ __device__ __forceinline__ void attend_wave(T* __restrict__ out_row, const T* __
   for (int c = lane; c < dk; c += 64) q_s[c] = ldf(q_row + c) * scale;
   __syncthreads();  // one wave per workgroup: orders the LDS writes before the other lanes' reads
   float m = sink ? sink_z : -INFINITY, l = sink ? 1.f : 0.f;  // the sink: one term exp(sink_z - m)
-  float acc[kMaxVC];
+  float acc[kGenVC];
 #pragma unroll
-  for (int c = 0; c < kMaxVC; ++c) acc[c] = 0.f;
+  for (int c = 0; c < kGenVC; ++c) acc[c] = 0.f;
   const long krow = (long)G * dk, vrow = (long)G * dv;
   for (int j0 = lo; j0 < hi; j0 += 64) {
     const int j = j0 + lane;
@@ -78,7 +80,7 @@ __device__ __forceinline__ void attend_wave(T* __restrict__ out_row, const T* __
     __syncthreads();
     const int n = min(64, hi - j0);
 #pragma unroll
-    for (int c = 0; c < kMaxVC; ++c) {
+    for (int c = 0; c < kGenVC; ++c) {
       const int dcol = lane + 64 * c;
       float a = acc[c] * alpha;
       if (dcol < dv)
@@ -91,7 +93,7 @@ __device__ __forceinline__ void attend_wave(T* __restrict__ out_row, const T* __
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-  for (int c = 0; c < kMaxVC; ++c) {
+  for (int c = 0; c < kGenVC; ++c) {
     const int dcol = lane + 64 * c;
     if (dcol < dv) stf(out_row + dcol, acc[c] * inv);
   }
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(64) void window_prefill_kernel(T* __restrict__ out,
                                                             const int* __restrict__ block_tables, int bt_stride, int S,
                                                             int Hq, int G, int dk, int dv, int bs, float scale,
                                                             int window, int sink, const float* __restrict__ sinks) {
-  __shared__ float q_s[kMaxDK];
+  __shared__ float q_s[kGenDK];
   __shared__ float p_s[64];
   const int r = blockIdx.x, h = blockIdx.y;
   const int s = find_segment(cu, S, r);
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(64) void window_decode_kernel(T* __restrict__ out, 
                                                            const int* __restrict__ seq_lens, int Hq, int G, int dk,
                                                            int dv, int bs, float scale, int window, int sink,
                                                            const float* __restrict__ sinks) {
-  __shared__ float q_s[kMaxDK];
+  __shared__ float q_s[kGenDK];
   __shared__ float p_s[64];
   const int b = blockIdx.x, h = blockIdx.y;
   const int n = seq_lens[b];
@@ -458,7 +460,7 @@ int k8sllm_hy_window_prefill(void* out, const void* qkv, long q_stride, const vo
                              int Hq, int G, int dk, int dv, int bs, float scale, int window, int sink,
                              const float* sinks, int f32, int mfma, hipStream_t s) {
   if (T <= 0 || S <= 0) return 0;
-  if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
+  if (dk > kGenDK || dv > 64 * kGenVC || G < 1 || Hq % G) return -1;
   // bf16 with matrix-core head sizes and 16-byte aligned rows: the MFMA kernel
   if (!f32 && mfma && bs == 16 && q_stride % 8 == 0 && (dk == 64 || dk == 128) && (dv == 64 || dv == 128)) {
     // query rows per wave: 32 once the step is large enough to fill the chip that way (two row tiles
@@ -498,9 +500,10 @@ int k8sllm_hy_window_decode(void* out, const void* qkv, long q_stride, const voi
                             int dv, int bs, float scale, int window, int sink, const float* sinks, int f32, int vec,
                             hipStream_t s) {
   if (B <= 0) return 0;
-  if (dk > kMaxDK || dv > 64 * kMaxVC || G < 1 || Hq % G) return -1;
+  if (dk > kGenDK || dv > 64 * kGenVC || G < 1 || Hq % G) return -1;
   const int R = Hq / G;
-  if (!f32 && vec && bs == 16 && dk % 8 == 0 && q_stride % 8 == 0 && (R == 1 || R == 2 || R == 4 || R == 8)) {
+  if (!f32 && vec && bs == 16 && dk % 8 == 0 && q_stride % 8 == 0 && dk <= kMaxDK && dv <= 64 * kMaxVC &&
+      (R == 1 || R == 2 || R == 4 || R == 8)) {
 #define K8SLLM_WD(RR)                                                                                                  \
   hipLaunchKernelGGL((window_decode_vec_kernel<RR, (RR == 8 ? 4 : 8)>), dim3(B, G), dim3(RR == 8 ? 256 : 512), 0, s,     \
                      (bf16_t*)out, (const bf16_t*)qkv,                                                                  \

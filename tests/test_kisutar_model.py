@@ -73,6 +73,17 @@ def test_single_mechanism_whole_prompt(layers):
     close(rig.run_cut("a", t, [45]), O.forward(cfg, rig.w, t))
 
 
+def test_odd_sizes_everywhere():
+    """Widths, ranks and head sizes that are multiples of nothing (rotated sizes stay even)."""
+    cfg = make_cfg([lat(3, 5, 2, 3, 9, 7, 6, 0.4, mlp=dense(11)), lat(5, 3, 2, 7, 5, 7, 11, 0.3, kv_from=0, mlp=moe(3, 2, 5, 9)),
+                    lat(1, 7, 4, 5, 3, 13, 4, 0.5, mlp=moe(7, 2, 3, 0))], width=37, vocab=53)
+    rig = rig_for(cfg, 31)
+    t = toks(41, 53, 3)
+    want = O.forward(cfg, rig.w, t)
+    for cuts in ([41], [3, 2, 17], [1]):
+        close(rig.run_cut("a", t, cuts), want)
+
+
 def test_layer_outputs_match_oracle():
     rig = rig_for(FULL, 5)
     t = toks(19, FULL["vocab"], 3)
@@ -455,6 +466,23 @@ def test_gpu_window_edges_and_sinks(win):
     want = _check_edge(cfg, w, t, far, win)
     for cuts in ([len(t)], [far + 1], [2] * ((far + win) // 2)):
         close(rig_for(cfg, w=w, device="cuda").run_cut("a", t, cuts), want, tol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gpu_odd_and_large_sizes(dtype):
+    """Sizes that are multiples of nothing, and a latent wider than the vector and matrix-core
+    kernels take (the any-size kernels)."""
+    odd = make_cfg([lat(3, 5, 2, 3, 9, 7, 6, 0.4, mlp=dense(11)), lat(5, 3, 2, 7, 5, 7, 11, 0.3, kv_from=0, mlp=moe(3, 2, 5, 9)),
+                    lat(1, 7, 4, 5, 3, 13, 4, 0.5, mlp=moe(7, 2, 3, 0))], width=37, vocab=53)
+    wide = make_cfg([lat(2, 8, 8, 8, 16, 328, 20, 0.3, mlp=dense(24))], width=48, vocab=53)
+    for cfg in (odd, wide):
+        rig = rig_for(cfg, 31, device="cuda", dtype=dtype)
+        t = toks(41, 53, 3)
+        want = O.forward(cfg, rig.w, t)
+        for cuts in ([41], [3, 2, 17]):
+            got = rig.run_cut("a", t, cuts)
+            close(got, want) if dtype == torch.float32 else close_most(got, want, 0.06, frac=0.85)
 
 
 @pytest.mark.gpu
