@@ -116,6 +116,31 @@ __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out
 // differ by one key at each end).
 // KS_MAX / DT_MAX bound the key width / 32 and the value width / 16 (register arrays); the real
 // widths are run-time (wave-uniform guards).  cu == nullptr: one row per sequence at seq_lens - 1.
+// how far (base-2 logits) a tile's maximum must exceed the running one before that is moved
+constexpr float kLazy = 8.f;
+
+// The page ids of a row's window, one per lane (64 tiles at a time): the id of a tile is then a
+// v_readlane away instead of a memory round trip in front of every tile's loads.
+struct PageIds {
+  const int* bt;
+  int first, last, reg;
+  __device__ __forceinline__ void init(const int* table, int first_tile, int last_tile) {
+    bt = table;
+    first = first_tile;
+    last = last_tile;
+    reg = bt[min(first + (int)(threadIdx.x & 63), last)];
+  }
+  __device__ __forceinline__ long at(int j0) {  // j0: wave-uniform key position of a tile
+    int idx = __builtin_amdgcn_readfirstlane(j0 >> 4) - first;
+    if (idx >= 64) {  // windows of more than 1024 keys: the next 64 ids
+      first += idx & ~63;
+      reg = bt[min(first + (int)(threadIdx.x & 63), last)];
+      idx &= 63;
+    }
+    return (long)__builtin_amdgcn_readlane(reg, idx);
+  }
+};
+
 template <int KS_MAX, int DT_MAX, int NW, int QT, bool DB>
 __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache,
@@ -192,10 +217,12 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
   const bf16_t* vbase = v_cache + (long)c16 * 16 + 4 * quad;
   const long vpage = (long)dv * 16;
   const int jfirst = (lo & ~15) + 16 * wave;
+  PageIds pages;
+  pages.init(bt, lo >> 4, (hi - 1) >> 4);
   bf16x8 kf_n[KS_MAX];
   s16x4 vf_n[DT_MAX];
   auto issue = [&](int j0) {
-    const long pg = bt[j0 >> 4];
+    const long pg = pages.at(j0);
     const bf16_t* krow = kbase + ((pg << 4) + (min(j0 + c16, hi - 1) & 15)) * dkp;
 #pragma unroll
     for (int ks = 0; ks < KS_MAX; ++ks)
@@ -228,20 +255,30 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
         if (ks < nks) sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[t][ks], sacc, 0, 0, 0);
       const int pt = p0 + t, lot = window > 0 ? max(0, pt - window + 1) : 0;
       float sv[4], tmax = -INFINITY;
+      if (t < nt && j0 >= lot && j0 + 15 <= pt) {  // wave-uniform: every key of the tile is live
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, head c16
-        const int j = j0 + 4 * quad + i;
-        sv[i] = (t < nt && j >= lot && j <= pt) ? sacc[i] * sc2 : -INFINITY;
-        tmax = fmaxf(tmax, sv[i]);
+        for (int i = 0; i < 4; ++i) {
+          sv[i] = sacc[i] * sc2;
+          tmax = fmaxf(tmax, sv[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {  // sacc[i]: key j0 + 4 quad + i, head c16
+          const int j = j0 + 4 * quad + i;
+          sv[i] = (t < nt && j >= lot && j <= pt) ? sacc[i] * sc2 : -INFINITY;
+          tmax = fmaxf(tmax, sv[i]);
+        }
       }
       tmax = xor32_max_f(xor16_max(tmax));
-      const float mn = fmaxf(m[t], tmax);
-      // a tile may hold no live key of token t (QT > 1: the window's first or last tile): nothing moves
-      alpha[t] = (m[t] == -INFINITY || mn == -INFINITY) ? (mn == -INFINITY ? 1.f : 0.f) : __builtin_amdgcn_exp2f(m[t] - mn);
+      // the running maximum only moves when it is beaten by more than kLazy (weights then stay below
+      // 2^kLazy, harmless in fp32 sums): the rescale of the whole output accumulator becomes rare.
+      // A wave's first tile always holds a live key (QT == 1) or m starts finite (the sink), so mn is finite
+      const float mn = tmax > m[t] + kLazy ? tmax : m[t];
+      alpha[t] = __builtin_amdgcn_exp2f(m[t] - mn);
       float ps = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = sv[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sv[i] - mn);
+        const float pv = __builtin_amdgcn_exp2f(sv[i] - mn);
         ps += pv;
         pb[t][i] = (short)f2bf(pv);
       }
@@ -314,6 +351,209 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
   }
 }
 
+// Prompt chunks of large steps: the same tiles with the 16-key page staged ONCE per workgroup in LDS.
+// A workgroup is 4 waves x QT consecutive tokens of one segment (x 16 heads); a key tile is one page,
+// i.e. one contiguous block of the key pages and one of the value pages, so staging is two straight
+// copies with 16-byte loads (the next three pages' loads are in flight while this one is computed,
+// two LDS buffers, one barrier per tile).  LDS rows are padded (keys: + 8 elements, values: 16 tokens + 4) so
+// that the fragment reads of a quarter wave fall on different banks.  Every wave starts from the sink.
+template <int KS_MAX, int DT_MAX, int QT>
+__global__ __launch_bounds__(256) void latent_attn_lds_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
+    const int* __restrict__ block_tables, int bt_stride, int S, int H, int dkp, int dv, float scale, int window,
+    const float* __restrict__ sinks) {
+  constexpr int TW = 4 * QT;           // tokens per workgroup
+  constexpr int KP = KS_MAX * 32 + 8;  // LDS pitch of a key row (elements)
+  constexpr int VP = 20;               // LDS pitch of a value dim's 16 tokens
+  constexpr int KC = (KS_MAX * 32 * 2 + 255) / 256, VC = (DT_MAX * 16 * 2 + 255) / 256;  // 16-byte pieces per thread
+  __shared__ __attribute__((aligned(16))) bf16_t k_s[2][16 * KP];
+  __shared__ __attribute__((aligned(16))) bf16_t v_s[2][DT_MAX * 16 * VP];
+  const float sc2 = scale * 1.44269504088896341f;
+  const int nwg = gridDim.x * gridDim.y, lin = blockIdx.y * gridDim.x + blockIdx.x;
+  const int xcd = lin & 7, glin = xcd * (nwg >> 3) + min(xcd, nwg & 7) + (lin >> 3);  // see latent_attn_mfma_kernel
+  const int hg = glin % (int)gridDim.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c16 = lane & 15, quad = lane >> 4;
+  int s = 0, g = glin / (int)gridDim.y, n = 0;
+  for (; s < S; ++s) {  // token groups are numbered segment by segment
+    n = cu[s + 1] - cu[s];
+    const int ng = (n + TW - 1) / TW;
+    if (g < ng) break;
+    g -= ng;
+  }
+  if (s >= S) return;
+  const int nt = min(TW, n - g * TW);             // live tokens of the group
+  const int row0 = cu[s] + g * TW, p0 = ctx[s] + g * TW;
+  const int nh = min(16, H - hg * 16);
+  const int nks = dkp >> 5, ndt = dv >> 4;
+  const int head = hg * 16 + min(c16, nh - 1);
+  const int* bt = block_tables + (long)s * bt_stride;
+  const int lo = window > 0 ? max(0, p0 - window + 1) : 0, hi = p0 + nt;
+  const int tok0 = wave * QT;                     // this wave's first token in the group
+  const bool wave_live = tok0 < nt;
+  bf16x8 qf[QT][KS_MAX];
+  f32x4 oacc[QT][DT_MAX];
+  float m[QT], l[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const bf16_t* qrow = q + (long)(row0 + min(tok0 + t, nt - 1)) * q_stride + (long)head * dkp + 8 * quad;
+#pragma unroll
+    for (int ks = 0; ks < KS_MAX; ++ks)
+      if (ks < nks) qf[t][ks] = *reinterpret_cast<const bf16x8*>(qrow + 32 * ks);
+#pragma unroll
+    for (int dt = 0; dt < DT_MAX; ++dt) oacc[t][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m[t] = sinks != nullptr ? sinks[head] * 1.44269504088896341f : 0.f;
+    l[t] = 1.f;
+  }
+  // staging: piece c of the page's keys is 8 elements of row c / (dkp / 8); piece c of its values is
+  // tokens 8 (c & 1) .. of dim c / 2.  The LDS offsets of a thread's pieces never change.
+  const int nkc = 2 * dkp, nvc = 2 * dv, kpr = dkp >> 3;
+  int k_off[KC], v_off[VC];
+#pragma unroll
+  for (int i = 0; i < KC; ++i) {
+    const int c = tid + 256 * i;
+    k_off[i] = c < nkc ? (c / kpr) * KP + (c % kpr) * 8 : -1;
+  }
+#pragma unroll
+  for (int i = 0; i < VC; ++i) {
+    const int c = tid + 256 * i;
+    v_off[i] = c < nvc ? (c >> 1) * VP + (c & 1) * 8 : -1;
+  }
+  PageIds pages;
+  pages.init(bt, lo >> 4, (hi - 1) >> 4);
+  // three register sets keep the pages of the next three tiles in flight (one tile of compute does not
+  // cover a load's latency); a set is written to the idle LDS buffer one tile before its use and
+  // refilled at once
+  uint4 kr0[KC], vr0[VC], kr1[KC], vr1[VC], kr2[KC], vr2[VC];
+  auto stage_load = [&](uint4 (&kreg)[KC], uint4 (&vreg)[VC], int j0) {
+    if (j0 >= hi) return;
+    const long pg = pages.at(j0);
+    const uint4* ksrc = reinterpret_cast<const uint4*>(k_cache + pg * 16 * dkp);
+    const uint4* vsrc = reinterpret_cast<const uint4*>(v_cache + pg * 16 * dv);
+#pragma unroll
+    for (int i = 0; i < KC; ++i)
+      if (k_off[i] >= 0) kreg[i] = ksrc[tid + 256 * i];
+#pragma unroll
+    for (int i = 0; i < VC; ++i)
+      if (v_off[i] >= 0) vreg[i] = vsrc[tid + 256 * i];
+  };
+  auto stage_store = [&](int b, const uint4 (&kreg)[KC], const uint4 (&vreg)[VC]) {
+#pragma unroll
+    for (int i = 0; i < KC; ++i)
+      if (k_off[i] >= 0) *reinterpret_cast<uint4*>(&k_s[b][k_off[i]]) = kreg[i];
+#pragma unroll
+    for (int i = 0; i < VC; ++i)
+      if (v_off[i] >= 0) {  // 8-byte aligned rows: two halves
+        *reinterpret_cast<uint2*>(&v_s[b][v_off[i]]) = make_uint2(vreg[i].x, vreg[i].y);
+        *reinterpret_cast<uint2*>(&v_s[b][v_off[i] + 4]) = make_uint2(vreg[i].z, vreg[i].w);
+      }
+  };
+  const int jfirst = lo & ~15;
+  stage_load(kr0, vr0, jfirst);
+  stage_load(kr1, vr1, jfirst + 16);
+  stage_load(kr2, vr2, jfirst + 32);
+  stage_store(0, kr0, vr0);
+  stage_load(kr0, vr0, jfirst + 48);
+  __syncthreads();
+  int buf = 0;
+  // one tile: compute from LDS buffer ``buf``, then hand the next tile (held in nk / nv) to the other buffer
+  auto tile = [&](int j0, uint4 (&nk)[KC], uint4 (&nv)[VC]) {
+    if (wave_live) {
+      const bf16_t* ks_ = &k_s[buf][c16 * KP + 8 * quad];
+      const bf16_t* vs_ = &v_s[buf][c16 * VP + 4 * quad];
+      f32x4 sacc[QT];
+#pragma unroll
+      for (int t = 0; t < QT; ++t) sacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS_MAX; ++ks)
+        if (ks < nks) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks_ + 32 * ks);
+#pragma unroll
+          for (int t = 0; t < QT; ++t) sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][ks], sacc[t], 0, 0, 0);
+        }
+      s16x4 pb[QT];
+      float alpha[QT];
+      bool rescale[QT];
+#pragma unroll
+      for (int t = 0; t < QT; ++t) {
+        const int pt = p0 + tok0 + t, lot = window > 0 ? max(0, pt - window + 1) : 0;
+        const bool tl = tok0 + t < nt;
+        float sv[4], tmax = -INFINITY;
+        if (tl && j0 >= lot && j0 + 15 <= pt) {  // wave-uniform: every key of the tile is live
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            sv[i] = sacc[t][i] * sc2;
+            tmax = fmaxf(tmax, sv[i]);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {  // sacc[t][i]: key j0 + 4 quad + i, head c16
+            const int j = j0 + 4 * quad + i;
+            sv[i] = (tl && j >= lot && j <= pt) ? sacc[t][i] * sc2 : -INFINITY;
+            tmax = fmaxf(tmax, sv[i]);
+          }
+        }
+        tmax = xor32_max_f(xor16_max(tmax));
+        const float mn = tmax > m[t] + kLazy ? tmax : m[t];  // m is finite from the start (the sink)
+        alpha[t] = __builtin_amdgcn_exp2f(m[t] - mn);
+        float ps = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pv = __builtin_amdgcn_exp2f(sv[i] - mn);
+          ps += pv;
+          pb[t][i] = (short)f2bf(pv);
+        }
+        ps = xor32_sum_f(xor16_sum(ps));
+        l[t] = l[t] * alpha[t] + ps;
+        m[t] = mn;
+        rescale[t] = __any(alpha[t] != 1.f);
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT_MAX; ++dt)
+        if (dt < ndt) {
+          const s16x4 vf = *reinterpret_cast<const s16x4*>(vs_ + dt * 16 * VP);
+#pragma unroll
+          for (int t = 0; t < QT; ++t) {
+            if (rescale[t]) {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
+            }
+            oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pb[t], oacc[t][dt], 0, 0, 0);
+          }
+        }
+    }
+    if (j0 + 16 < hi) {
+      stage_store(buf ^ 1, nk, nv);
+      stage_load(nk, nv, j0 + 64);
+    }
+    __syncthreads();
+    buf ^= 1;
+  };
+  for (int j0 = jfirst;;) {
+    tile(j0, kr1, vr1);
+    if ((j0 += 16) >= hi) break;
+    tile(j0, kr2, vr2);
+    if ((j0 += 16) >= hi) break;
+    tile(j0, kr0, vr0);
+    if ((j0 += 16) >= hi) break;
+  }
+  if (!wave_live || c16 >= nh) return;
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    if (tok0 + t >= nt) break;
+    const float inv = l[t] > 0.f ? 1.f / l[t] : 0.f;
+    bf16_t* orow = out + ((long)(row0 + tok0 + t) * H + hg * 16 + c16) * dv;
+#pragma unroll
+    for (int dt = 0; dt < DT_MAX; ++dt)
+      if (dt < ndt) {
+        uint2 w;
+        w.x = pack2(oacc[t][dt][0] * inv, oacc[t][dt][1] * inv);
+        w.y = pack2(oacc[t][dt][2] * inv, oacc[t][dt][3] * inv);
+        *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * quad) = w;
+      }
+  }
+}
+
 }  // namespace k8sllm
 
 using namespace k8sllm;
@@ -358,11 +598,27 @@ int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const vo
   if (bs != 16 || dkp % 32 || dv % 16 || dkp > 320 || dv > 256 || q_stride % 8) return 1;
   const unsigned hgs = (unsigned)((H + 15) / 16);
   // split 1 / 4 force that many waves with one token each (tests, measurements); 2: two tokens per wave
-  // prompt chunks: two tokens per wave, no register double buffer (two waves per SIMD hide each
-  // other's loads better than one wave hides its own: measured); few rows: eight waves per token.
-  // split: 1 / 2 tokens per wave, 4 / 8 waves per token; + 16: with the register double buffer
+  // prompt chunks of small steps: two tokens per wave, no register double buffer (two waves per SIMD
+  // hide each other's loads better than one wave hides its own: measured); few rows: eight waves per token.
+  // split: 1 / 2 tokens per wave, 4 / 8 waves per token; + 16: with the register double buffer; 32 / 33:
+  // the LDS-staged kernel with two / one token per wave (prompt chunks only)
   const bool big = T * hgs >= 2048;
-  const bool db = split >= 16;
+  if (cu != nullptr && (split == 32 || split == 33 || (split == 0 && big))) {  // prompt chunks of a large step: pages staged in LDS
+    const int qt = split == 32 ? 2 : 1;  // tokens per wave: one measured faster (more waves per SIMD)
+    const dim3 grid((unsigned)(T / (4 * qt) + S), hgs);
+#define K8SLLM_LL(KS, DT, QT)                                                                                          \
+  hipLaunchKernelGGL((latent_attn_lds_kernel<KS, DT, QT>), grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)q,        \
+                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, block_tables, bt_stride, S, H,  \
+                     dkp, dv, scale, window, sinks)
+    if (dkp <= 128 && dv <= 128) {
+      if (qt == 1) K8SLLM_LL(4, 8, 1); else K8SLLM_LL(4, 8, 2);
+    } else {
+      if (qt == 1) K8SLLM_LL(10, 16, 1); else K8SLLM_LL(10, 16, 2);
+    }
+#undef K8SLLM_LL
+    return (int)hipGetLastError();
+  }
+  const bool db = split >= 16 && split < 32;
   if (db) split -= 16;
   if (split != 0 && split != 1 && split != 2 && split != 4 && split != 8) return -1;
   const int nw = split == 4 || split == 8 ? split : ((split == 1 || split == 2 || big) ? 1 : 8);
