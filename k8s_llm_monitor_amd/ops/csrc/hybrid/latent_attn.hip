@@ -141,7 +141,7 @@ struct PageIds {
   }
 };
 
-template <int KS_MAX, int DT_MAX, int NW, int QT, bool DB>
+template <int KS_MAX, int DT_MAX, int NW, int QT>
 __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ cu, const int* __restrict__ ctx,
@@ -232,18 +232,16 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
     for (int dt = 0; dt < DT_MAX; ++dt)
       if (dt < ndt) vf_n[dt] = *reinterpret_cast<const s16x4*>(vpg + dt * 256);
   };
-  // DB: the next tile's fragments are in flight while this one is computed (one wave per SIMD hides
-  // its own latency); else fewer registers and more waves per SIMD hide each other's
-  if (DB && jfirst < hi) issue(jfirst);
+  // no register double buffer: with fewer registers two waves fit a SIMD and hide each other's loads
+  // better than one wave hides its own (measured both ways)
   for (int j0 = jfirst; j0 < hi; j0 += 16 * NW) {
     bf16x8 kf[KS_MAX];
     s16x4 vf[DT_MAX];
-    if (!DB) issue(j0);
+    issue(j0);
 #pragma unroll
     for (int ks = 0; ks < KS_MAX; ++ks) kf[ks] = kf_n[ks];
 #pragma unroll
     for (int dt = 0; dt < DT_MAX; ++dt) vf[dt] = vf_n[dt];
-    if (DB && j0 + 16 * NW < hi) issue(j0 + 16 * NW);
     s16x4 pb[QT];
     float alpha[QT];
     bool rescale[QT];
@@ -287,17 +285,22 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(
       m[t] = mn;
       rescale[t] = __any(alpha[t] != 1.f);
     }
+    // the rescale of a token's whole accumulator is ONE block behind one wave-uniform branch (a branch
+    // around each tile's four multiplies is flattened by the compiler into multiplies on every tile)
+#pragma unroll
+    for (int t = 0; t < QT; ++t)
+      if (rescale[t]) {
+#pragma unroll
+        for (int dt = 0; dt < DT_MAX; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
+      }
 #pragma unroll
     for (int dt = 0; dt < DT_MAX; ++dt)
       if (dt < ndt) {
 #pragma unroll
-        for (int t = 0; t < QT; ++t) {
-          if (rescale[t]) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
-          }
+        for (int t = 0; t < QT; ++t)
           oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[dt], pb[t], oacc[t][dt], 0, 0, 0);
-        }
       }
   }
   // oacc[t][dt][i] = O[token t][head c16][d = 16 dt + 4 quad + i]
@@ -509,17 +512,20 @@ __global__ __launch_bounds__(256) void latent_attn_lds_kernel(
         rescale[t] = __any(alpha[t] != 1.f);
       }
 #pragma unroll
+      for (int t = 0; t < QT; ++t)
+        if (rescale[t]) {  // one block for the whole accumulator (see latent_attn_mfma_kernel)
+#pragma unroll
+          for (int dt = 0; dt < DT_MAX; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
+        }
+#pragma unroll
       for (int dt = 0; dt < DT_MAX; ++dt)
         if (dt < ndt) {
           const s16x4 vf = *reinterpret_cast<const s16x4*>(vs_ + dt * 16 * VP);
 #pragma unroll
-          for (int t = 0; t < QT; ++t) {
-            if (rescale[t]) {
-#pragma unroll
-              for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
-            }
+          for (int t = 0; t < QT; ++t)
             oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pb[t], oacc[t][dt], 0, 0, 0);
-          }
         }
     }
     if (j0 + 16 < hi) {
@@ -597,14 +603,12 @@ int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const vo
   if (T <= 0) return 0;
   if (bs != 16 || dkp % 32 || dv % 16 || dkp > 320 || dv > 256 || q_stride % 8) return 1;
   const unsigned hgs = (unsigned)((H + 15) / 16);
-  // split 1 / 4 force that many waves with one token each (tests, measurements); 2: two tokens per wave
-  // prompt chunks of small steps: two tokens per wave, no register double buffer (two waves per SIMD
-  // hide each other's loads better than one wave hides its own: measured); few rows: eight waves per token.
-  // split: 1 / 2 tokens per wave, 4 / 8 waves per token; + 16: with the register double buffer; 32 / 33:
-  // the LDS-staged kernel with two / one token per wave (prompt chunks only)
-  const bool big = T * hgs >= 2048;
-  if (cu != nullptr && (split == 32 || split == 33 || (split == 0 && big))) {  // prompt chunks of a large step: pages staged in LDS
-    const int qt = split == 32 ? 2 : 1;  // tokens per wave: one measured faster (more waves per SIMD)
+  // The launcher's choice (split 0): prompt chunks of a large step take the LDS-staged kernel with one
+  // token per wave; small steps and decoding eight waves per token (a row's window is its only
+  // parallel axis).  Forced (tests, measurements): 1 / 2 tokens per wave with fragments from global
+  // memory, 4 / 8 waves per token, 32 / 33 the LDS-staged kernel with two / one token per wave.
+  if (cu != nullptr && (split == 32 || split == 33 || (split == 0 && T * hgs >= 2048))) {
+    const int qt = split == 32 ? 2 : 1;  // one token per wave measured faster (more waves per SIMD)
     const dim3 grid((unsigned)(T / (4 * qt) + S), hgs);
 #define K8SLLM_LL(KS, DT, QT)                                                                                          \
   hipLaunchKernelGGL((latent_attn_lds_kernel<KS, DT, QT>), grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)q,        \
@@ -618,24 +622,19 @@ int k8sllm_hy_latent_attention(void* out, const void* q, long q_stride, const vo
 #undef K8SLLM_LL
     return (int)hipGetLastError();
   }
-  const bool db = split >= 16 && split < 32;
-  if (db) split -= 16;
   if (split != 0 && split != 1 && split != 2 && split != 4 && split != 8) return -1;
-  const int nw = split == 4 || split == 8 ? split : ((split == 1 || split == 2 || big) ? 1 : 8);
-  const int qt = (cu != nullptr && nw == 1 && split != 1) ? 2 : 1;
+  const int nw = split == 4 || split == 8 ? split : ((split == 1 || split == 2) ? 1 : 8);
+  const int qt = (cu != nullptr && split == 2) ? 2 : 1;
   const dim3 grid((unsigned)(qt == 1 ? T : T / qt + S), hgs);
-#define K8SLLM_LA(KS, DT, NW, QT, DB)                                                                                  \
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<KS, DT, NW, QT, DB>), grid, dim3(64 * NW), 0, s, (bf16_t*)out,            \
+#define K8SLLM_LA(KS, DT, NW, QT)                                                                                      \
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KS, DT, NW, QT>), grid, dim3(64 * NW), 0, s, (bf16_t*)out,                \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, cu, ctx, seq_lens,     \
                      block_tables, bt_stride, S, H, dkp, dv, scale, window, sinks)
 #define K8SLLM_LAS(KS, DT)                                            \
-  if (nw == 8) K8SLLM_LA(KS, DT, 8, 1, false);                        \
-  else if (nw == 4 && db) K8SLLM_LA(KS, DT, 4, 1, true);              \
-  else if (nw == 4) K8SLLM_LA(KS, DT, 4, 1, false);                   \
-  else if (qt == 2 && db) K8SLLM_LA(KS, DT, 1, 2, true);              \
-  else if (qt == 2) K8SLLM_LA(KS, DT, 1, 2, false);                   \
-  else if (db) K8SLLM_LA(KS, DT, 1, 1, true);                         \
-  else K8SLLM_LA(KS, DT, 1, 1, false)
+  if (nw == 8) K8SLLM_LA(KS, DT, 8, 1);                               \
+  else if (nw == 4) K8SLLM_LA(KS, DT, 4, 1);                          \
+  else if (qt == 2) K8SLLM_LA(KS, DT, 1, 2);                          \
+  else K8SLLM_LA(KS, DT, 1, 1)
   if (dkp <= 128 && dv <= 128) { K8SLLM_LAS(4, 8); }
   else { K8SLLM_LAS(10, 16); }
 #undef K8SLLM_LAS

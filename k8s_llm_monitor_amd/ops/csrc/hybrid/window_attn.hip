@@ -409,17 +409,22 @@ __global__ __launch_bounds__(64) void window_prefill_mfma_kernel(
       m[t] = mn;
       rescale[t] = __any(alpha[t] != 1.f);
     }
+    // wave-uniform: once the running maxima settle, most tiles skip the rescale.  ONE block for a
+    // row tile's whole accumulator: a branch around each value tile's four multiplies is flattened by
+    // the compiler into multiplies on every tile
+#pragma unroll
+    for (int t = 0; t < QT; ++t)
+      if (rescale[t]) {
+#pragma unroll
+        for (int dt = 0; dt < DV / 16; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
+      }
 #pragma unroll
     for (int dt = 0; dt < DV / 16; ++dt) {
       const s16x4 a = vf[dt];
 #pragma unroll
-      for (int t = 0; t < QT; ++t) {
-        if (rescale[t]) {  // wave-uniform: once the running maxima settle, most tiles skip this
-#pragma unroll
-          for (int i = 0; i < 4; ++i) oacc[t][dt][i] *= alpha[t];
-        }
-        oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[t], oacc[t][dt], 0, 0, 0);
-      }
+      for (int t = 0; t < QT; ++t) oacc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[t], oacc[t][dt], 0, 0, 0);
     }
   }
 #pragma unroll

@@ -352,9 +352,9 @@ def latent_attention(qa: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     chunks (rows of segment s at positions ctx[s] ..); else ``seq_lens``: one row per sequence, at its
     newest token.  Returns [T, H * kv_rank].  GPU, bf16, pitch a multiple of 32 up to 320 and kv_rank a
     multiple of 16 up to 256 (``fast``): the matrix-core kernel, 16 heads of one token per tile
-    (``split`` 1: one wave per token, 2: two tokens of a chunk per wave, 4 / 8: that many waves share
-    a token's window, + 16: with the register double buffer, 32 / 33: pages staged in LDS for eight /
-    four tokens of a chunk at a time; 0: by the step's size - large steps' chunks take 33, few rows 8); other sizes and fp32:
+    (``split`` 1 / 2: one wave per one / two tokens, 4 / 8: that many waves share a token's window,
+    32 / 33: pages staged in LDS for eight / four tokens of a chunk at a time; 0: by the step's size -
+    large steps' chunks take 33, few rows 8); other sizes and fp32:
     the any-size kernels with one shared key/value head."""
     T, pitch, dv = qa.shape[0], k_cache.shape[2], v_cache.shape[2]
     if qa.is_cuda and fast and qa.dtype == torch.bfloat16:
