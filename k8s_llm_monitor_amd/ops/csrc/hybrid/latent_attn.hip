@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void latent_queries_kernel(T* __restrict__ out
 constexpr float kLazy = 8.f;
 
 // The page ids of a row's window, one per lane (64 tiles at a time): the id of a tile is then a
-// v_readlane away instead of a memory round trip in front of every tile's loads.
+// v_readlane away instead of a dependent memory access in front of every tile's loads.
 struct PageIds {
   const int* bt;
   int first, last, reg;
